@@ -1,4 +1,4 @@
-"""One registry from an architecture's name (config.json `architectures[0]`) to
+"""One registry from an architecture's name (config.json `architectures[0]`, or `architecture`) to
 its typed configuration, and through `to_spec()` to its model.  A configuration
 class offers `from_dict(config_json) -> cfg`, `cfg.to_dict()`, `cfg.to_spec()
 -> ModelSpec` and optionally `cfg.with_window(n)`."""
@@ -6,6 +6,7 @@ import json
 import os
 
 from .llama import ConfigError, LlamaConfig
+from .situlorn import SitulornConfig
 
 _ARCHITECTURES = {}
 
@@ -27,7 +28,7 @@ def registered_architectures():
 def config_from_dict(d):
     """The typed configuration of a config.json dictionary, chosen by its architecture."""
     archs = d.get("architectures") or []
-    name = archs[0] if archs else None
+    name = archs[0] if archs else d.get("architecture")
     if name not in _ARCHITECTURES:
         # convert.py:24-27: an unknown architecture is an error that lists the known ones
         raise ConfigError("architecture %r is not supported; registered: %s" % (name, registered_architectures()))
@@ -42,5 +43,6 @@ def config_from_folder(path):
         return config_from_dict(json.load(fh))
 
 
-for _name in LlamaConfig.ARCHITECTURES:
-    register_architecture(_name, LlamaConfig)
+for _cls in (LlamaConfig, SitulornConfig):
+    for _name in _cls.ARCHITECTURES:
+        register_architecture(_name, _cls)

@@ -1,0 +1,148 @@
+// Latent attention: keys and values of all heads are functions of one small vector c per token, so the
+// cache keeps one "head" a token, [rotated part | c | zeros up to the padded size], and attention runs in
+// the latent space: a query head becomes [its rotated part | W_uk_h^T q_h], the result of a head is a mix
+// of c vectors that W_uv_h turns into the head's values afterwards.  The attention kernels are the
+// grouped-query ones with one KV head.
+//
+//  * yalm_latent_pack: per token, the RMS norm of the down projection's first `rank` columns, and the
+//    head-shaped rows that the rotation kernel reads (query rotated parts scaled, key, value).
+//  * yalm_head_matmul: out[t, h, :] = scale * in[t, h, :] Wt[h] for every head, Wt [H, K, N]
+//    (optionally times sigmoid(gate)): the two per-head products (W_uk^T on queries, W_uv on results).
+//    float32 arithmetic; a workgroup owns a head and 16 tokens, a lane a column of the result.
+#include "common.h"
+#include "yalm_hip.h"
+
+namespace {
+
+constexpr int HM_TOK = 16;                 // tokens a workgroup
+constexpr int HM_THREADS = 256;
+constexpr int HM_KMAX = 512;               // the most K the LDS tile holds
+
+template <typename TI, typename TW, typename TO>
+__global__ __launch_bounds__(HM_THREADS) void head_matmul_kernel(const TI* __restrict__ in, long in_row, int in_head, int in_off,
+                                                                 const TW* __restrict__ wt, TO* __restrict__ out, long out_row,
+                                                                 int out_head, int out_off, float scale,
+                                                                 const float* __restrict__ gate, long gate_row, int T,
+                                                                 int K, int N) {
+  __shared__ float tile[HM_TOK][HM_KMAX];
+  const int h = blockIdx.y;
+  const int t0 = blockIdx.x * HM_TOK;
+  for (int i = threadIdx.x; i < HM_TOK * K; i += HM_THREADS) {
+    const int tt = i / K, k = i % K;
+    const int t = t0 + tt;
+    tile[tt][k] = t < T ? to_f32(in[(size_t)t * in_row + (size_t)h * in_head + in_off + k]) : 0.f;
+  }
+  __syncthreads();
+  const int tg = threadIdx.x / WAVE;        // a wave takes 4 of the 16 tokens
+  const int lane = threadIdx.x % WAVE;
+  const TW* w = wt + (size_t)h * K * N;
+  for (int n = lane; n < N; n += WAVE) {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < K; ++k) {
+      const float wv = to_f32(w[(size_t)k * N + n]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] += tile[tg * 4 + j][k] * wv;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int t = t0 + tg * 4 + j;
+      if (t >= T) continue;
+      float v = acc[j] * scale;
+      if (gate != nullptr) {
+        const float g = gate[(size_t)t * gate_row + (size_t)h * N + n];
+        v *= 1.0f / (1.0f + expf(-g));
+      }
+      out[(size_t)t * out_row + (size_t)h * out_head + out_off + n] = from_f32<TO>(v);
+    }
+  }
+}
+
+// One wave a (token, job).  job < H: the rotated part of query head `job`, scaled, and zeros behind the
+// latent part; job == H (has_kv only): the key and value rows.
+template <typename TN>
+__global__ __launch_bounds__(WAVE) void latent_pack_kernel(const float* __restrict__ proj, long proj_row, int q_head,
+                                                           int q_rot_off, int kv_off, const TN* __restrict__ norm_w, float eps,
+                                                           float q_scale, float* __restrict__ out, int H, int rot, int rank,
+                                                           int Dk, int has_kv) {
+  const int t = blockIdx.x, job = blockIdx.y, lane = threadIdx.x;
+  const float* row = proj + (size_t)t * proj_row;
+  float* dst = out + (size_t)t * (H + 2) * Dk;
+  if (job < H) {
+    float* q = dst + (size_t)job * Dk;
+    for (int i = lane; i < rot; i += WAVE) q[i] = row[(size_t)job * q_head + q_rot_off + i] * q_scale;
+    for (int i = rot + rank + lane; i < Dk; i += WAVE) q[i] = 0.f;
+    return;
+  }
+  if (!has_kv) return;
+  const float* d = row + kv_off;
+  float ss = 0.f;
+  for (int i = lane; i < rank; i += WAVE) ss += d[i] * d[i];
+  ss = wave_sum(ss);
+  const float s = 1.0f / sqrtf(ss / (float)rank + eps);
+  float* k = dst + (size_t)H * Dk;
+  float* v = k + Dk;
+  for (int i = lane; i < rot; i += WAVE) {
+    k[i] = d[rank + i];
+    v[i] = 0.f;
+  }
+  for (int i = lane; i < rank; i += WAVE) {
+    const float c = d[i] * s * to_f32(norm_w[i]);
+    k[rot + i] = c;
+    v[rot + i] = c;
+  }
+  for (int i = rot + rank + lane; i < Dk; i += WAVE) {
+    k[i] = 0.f;
+    v[i] = 0.f;
+  }
+}
+
+template <typename TI, typename TW, typename TO>
+int head_matmul_launch(const void* in, long in_row, int in_head, int in_off, const void* wt, void* out, long out_row,
+                       int out_head, int out_off, float scale, const float* gate, long gate_row, int T, int H, int K,
+                       int N, hipStream_t stream) {
+  dim3 grid(ceil_div(T, HM_TOK), H);
+  head_matmul_kernel<TI, TW, TO><<<grid, HM_THREADS, 0, stream>>>((const TI*)in, in_row, in_head, in_off, (const TW*)wt,
+                                                                  (TO*)out, out_row, out_head, out_off, scale, gate,
+                                                                  gate_row, T, K, N);
+  return launch_status();
+}
+
+}  // namespace
+
+extern "C" int yalm_head_matmul(const void* in, int in_dtype, long in_row, int in_head, int in_off, const void* wt,
+                                int w_dtype, void* out, int out_dtype, long out_row, int out_head, int out_off,
+                                float scale, const float* gate, long gate_row, int T, int H, int K, int N,
+                                hipStream_t stream) {
+  if (T <= 0) return YALM_OK;
+  if (H <= 0 || K <= 0 || N <= 0 || K > HM_KMAX || in_off < 0 || out_off < 0 || in_off + K > in_head ||
+      out_off + N > out_head || (long)H * in_head > in_row || (long)H * out_head > out_row ||
+      (gate != nullptr && (long)H * N > gate_row))
+    return YALM_ERR_ARG;
+#define HM(TI, TW, TO) \
+  return head_matmul_launch<TI, TW, TO>(in, in_row, in_head, in_off, wt, out, out_row, out_head, out_off, scale, gate, \
+                                        gate_row, T, H, K, N, stream)
+  if (in_dtype == YALM_F32 && w_dtype == YALM_F32 && out_dtype == YALM_F32) HM(float, float, float);
+  if (in_dtype == YALM_F32 && w_dtype == YALM_BF16 && out_dtype == YALM_F32) HM(float, bf16, float);
+  if (in_dtype == YALM_BF16 && w_dtype == YALM_BF16 && out_dtype == YALM_BF16) HM(bf16, bf16, bf16);
+#undef HM
+  return YALM_ERR_DTYPE;
+}
+
+extern "C" int yalm_latent_pack(const float* proj, long proj_row, int q_head, int q_rot_off, int kv_off,
+                                const void* norm_w, int norm_dtype, float eps, float q_scale, float* out, int T, int H,
+                                int rot, int rank, int Dk, int has_kv, hipStream_t stream) {
+  if (T <= 0) return YALM_OK;
+  if (H <= 0 || rot < 0 || rank <= 0 || Dk < rot + rank || q_rot_off < 0 || q_rot_off + rot > q_head ||
+      (long)H * q_head > proj_row || (has_kv && (norm_w == nullptr || kv_off < 0 || (long)kv_off + rank + rot > proj_row)))
+    return YALM_ERR_ARG;
+  dim3 grid(T, H + 1);
+  if (norm_dtype == YALM_BF16)
+    latent_pack_kernel<bf16><<<grid, WAVE, 0, stream>>>(proj, proj_row, q_head, q_rot_off, kv_off, (const bf16*)norm_w, eps,
+                                                        q_scale, out, H, rot, rank, Dk, has_kv);
+  else if (norm_dtype == YALM_F32)
+    latent_pack_kernel<float><<<grid, WAVE, 0, stream>>>(proj, proj_row, q_head, q_rot_off, kv_off, (const float*)norm_w,
+                                                         eps, q_scale, out, H, rot, rank, Dk, has_kv);
+  else
+    return YALM_ERR_DTYPE;
+  return launch_status();
+}

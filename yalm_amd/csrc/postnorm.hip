@@ -1,0 +1,108 @@
+// Kernels of layers that norm a sublayer's OUTPUT before it joins the residual stream
+// (x <- x + rms(y) * w), and of the PolyNorm activation.  Everything is float32 arithmetic on a row
+// per workgroup; inputs from GEMMs are float32, outputs go to the compute dtype.
+#include "common.h"
+#include "yalm_hip.h"
+
+namespace {
+
+constexpr int ROW_THREADS = 256;
+constexpr int ROW_WAVES = ROW_THREADS / WAVE;
+
+template <typename T>
+__global__ __launch_bounds__(ROW_THREADS) void cast_kernel(const float* __restrict__ x, T* __restrict__ out, long n) {
+  long i = (long)blockIdx.x * ROW_THREADS + threadIdx.x;
+  const long step = (long)gridDim.x * ROW_THREADS;
+  for (; i < n; i += step) out[i] = from_f32<T>(x[i]);
+}
+
+// x[r] += y[r] * rsqrt(mean(y[r]^2) + eps) * w; h[r] = T(x[r]) if h is given
+template <typename W, typename T>
+__global__ __launch_bounds__(ROW_THREADS) void norm_add_kernel(const float* __restrict__ y, const W* __restrict__ w, float eps,
+                                                               float* __restrict__ x, T* __restrict__ h, int D) {
+  __shared__ float red[ROW_WAVES];
+  const size_t row = (size_t)blockIdx.x * D;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < D; i += ROW_THREADS) {
+    const float v = y[row + i];
+    ss += v * v;
+  }
+  ss = block_sum<ROW_WAVES>(ss, red);
+  const float scale = 1.0f / sqrtf(ss / (float)D + eps);
+  for (int i = threadIdx.x; i < D; i += ROW_THREADS) {
+    const float v = x[row + i] + y[row + i] * scale * to_f32(w[i]);
+    x[row + i] = v;
+    if (h != nullptr) h[row + i] = from_f32<T>(v);
+  }
+}
+
+// out = a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps) over the row
+template <typename T>
+__global__ __launch_bounds__(ROW_THREADS) void polynorm_kernel(const float* __restrict__ z, const float* __restrict__ coef, float eps,
+                                                               T* __restrict__ out, int F) {
+  __shared__ float red[ROW_WAVES];
+  const size_t row = (size_t)blockIdx.x * F;
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+  for (int i = threadIdx.x; i < F; i += ROW_THREADS) {
+    const float v = z[row + i];
+    const float v2 = v * v;
+    s2 += v2;
+    s4 += v2 * v2;
+    s6 += v2 * v2 * v2;
+  }
+  s2 = block_sum<ROW_WAVES>(s2, red);
+  s4 = block_sum<ROW_WAVES>(s4, red);
+  s6 = block_sum<ROW_WAVES>(s6, red);
+  const float r1 = coef[0] / sqrtf(s2 / (float)F + eps);
+  const float r2 = coef[1] / sqrtf(s4 / (float)F + eps);
+  const float r3 = coef[2] / sqrtf(s6 / (float)F + eps);
+  const float e = coef[3];
+  for (int i = threadIdx.x; i < F; i += ROW_THREADS) {
+    const float v = z[row + i];
+    out[row + i] = from_f32<T>(v * r1 + v * v * r2 + v * v * v * r3 + e);
+  }
+}
+
+}  // namespace
+
+extern "C" int yalm_cast(const float* x, void* out, long n, int out_dtype, hipStream_t stream) {
+  if (n <= 0) return YALM_OK;
+  const int blocks = (int)((n + ROW_THREADS - 1) / ROW_THREADS < 4096 ? (n + ROW_THREADS - 1) / ROW_THREADS : 4096);
+  if (out_dtype == YALM_BF16)
+    cast_kernel<bf16><<<blocks, ROW_THREADS, 0, stream>>>(x, (bf16*)out, n);
+  else if (out_dtype == YALM_F32)
+    cast_kernel<float><<<blocks, ROW_THREADS, 0, stream>>>(x, (float*)out, n);
+  else
+    return YALM_ERR_DTYPE;
+  return launch_status();
+}
+
+extern "C" int yalm_norm_add(const float* y, const void* w, int w_dtype, float eps, float* x, void* h_out, int h_dtype,
+                             int R, int D, hipStream_t stream) {
+  if (R <= 0) return YALM_OK;
+  if (D <= 0) return YALM_ERR_ARG;
+  if (w_dtype != YALM_F32 && w_dtype != YALM_BF16) return YALM_ERR_DTYPE;
+  if (h_out != nullptr && h_dtype != YALM_F32 && h_dtype != YALM_BF16) return YALM_ERR_DTYPE;
+  const bool hb = h_out != nullptr && h_dtype == YALM_BF16;
+  if (w_dtype == YALM_F32) {
+    if (hb) norm_add_kernel<float, bf16><<<R, ROW_THREADS, 0, stream>>>(y, (const float*)w, eps, x, (bf16*)h_out, D);
+    else norm_add_kernel<float, float><<<R, ROW_THREADS, 0, stream>>>(y, (const float*)w, eps, x, (float*)h_out, D);
+  } else {
+    if (hb) norm_add_kernel<bf16, bf16><<<R, ROW_THREADS, 0, stream>>>(y, (const bf16*)w, eps, x, (bf16*)h_out, D);
+    else norm_add_kernel<bf16, float><<<R, ROW_THREADS, 0, stream>>>(y, (const bf16*)w, eps, x, (float*)h_out, D);
+  }
+  return launch_status();
+}
+
+extern "C" int yalm_polynorm(const float* z, const float* coef, float eps, void* out, int out_dtype, int R, int F,
+                             hipStream_t stream) {
+  if (R <= 0) return YALM_OK;
+  if (F <= 0) return YALM_ERR_ARG;
+  if (out_dtype == YALM_BF16)
+    polynorm_kernel<bf16><<<R, ROW_THREADS, 0, stream>>>(z, coef, eps, (bf16*)out, F);
+  else if (out_dtype == YALM_F32)
+    polynorm_kernel<float><<<R, ROW_THREADS, 0, stream>>>(z, coef, eps, (float*)out, F);
+  else
+    return YALM_ERR_DTYPE;
+  return launch_status();
+}

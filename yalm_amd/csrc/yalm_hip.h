@@ -237,6 +237,45 @@ int yalm_sample(const float* logits, const float* u, float temperature, int* out
 // prob[r] = softmax(logits[r, :])[index[r]] (src/sampler.cpp:11-25)
 int yalm_token_prob(const float* logits, const int* index, float* prob, int R, int V, hipStream_t stream);
 
+// Layers that norm a sublayer's OUTPUT before it joins the residual stream (postnorm.hip).
+// yalm_cast: out[i] = dtype(x[i]).  yalm_norm_add: x[r, :] += y[r, :] * rsqrt(mean(y[r]^2) + eps) * w, and if h_out is
+// given h_out[r, :] = dtype(x_new[r, :]) (the next sublayer's input).  yalm_polynorm: out[r, :] = a N(z) + b N(z^2) +
+// c N(z^3) + e with powers element by element, N(v) = v / sqrt(mean(v^2) + eps) over the row and coef = {a, b, c, e}
+// (float32, on the device).
+int yalm_cast(const float* x, void* out, long n, int out_dtype, hipStream_t stream);
+int yalm_norm_add(const float* y, const void* w, int w_dtype, float eps, float* x, void* h_out, int h_dtype, int R, int D,
+                  hipStream_t stream);
+int yalm_polynorm(const float* z, const float* coef, float eps, void* out, int out_dtype, int R, int F,
+                  hipStream_t stream);
+
+// Latent attention (latent.hip).  yalm_head_matmul: for every token t and head h,
+//   out[t * out_row + h * out_head + out_off + n] = scale * sum_k in[t * in_row + h * in_head + in_off + k] * wt[h, k, n]
+// (n < N, k < K <= 512), times sigmoid(gate[t * gate_row + h * N + n]) if gate (float32) is given.  Types (in, wt,
+// out): all float32; float32, bfloat16, float32; all bfloat16.
+// yalm_latent_pack fills out float32 [T, (H + 2) * Dk], the head-shaped rows that yalm_rope_kv_write reads with
+// H query heads and one KV head of size Dk = [rot | rank | zeros]: query head h gets q_scale * proj[t, h * q_head +
+// q_rot_off + i] in its first rot places and zeros behind rot + rank (the places between are the caller's, see
+// yalm_head_matmul); with has_kv the key row is [proj[t, kv_off + rank + i] | c | 0] and the value row [0 | c | 0], c =
+// proj[t, kv_off + i] * rsqrt(mean over the rank columns of their squares + eps) * norm_w[i].
+int yalm_head_matmul(const void* in, int in_dtype, long in_row, int in_head, int in_off, const void* wt, int w_dtype,
+                     void* out, int out_dtype, long out_row, int out_head, int out_off, float scale, const float* gate,
+                     long gate_row, int T, int H, int K, int N, hipStream_t stream);
+int yalm_latent_pack(const float* proj, long proj_row, int q_head, int q_rot_off, int kv_off, const void* norm_w,
+                     int norm_dtype, float eps, float q_scale, float* out, int T, int H, int rot, int rank, int Dk,
+                     int has_kv, hipStream_t stream);
+
+// Mixture of experts (moe.hip).  yalm_moe_route: ids, wts [T, top] = the `top` experts with the largest
+// softmax(w_router h) over all E experts (float32 arithmetic; the lowest index on ties) and those scores (renorm: divided
+// by their sum).  The pair kernels serve every (token, choice) pair from its expert's weights: w_gate, w_up [E, F, D],
+// w_down [E, D, F]; mid [T * top, F] = g sigmoid(alpha g) (u + 1) with g = min(w_gate h, limit), u = clamp(w_up h,
+// -limit, limit) (limit <= 0: unclamped); out float32 [T, D] = (accumulate: out +) sum_k wts[t, k] * w_down[ids[t, k]] mid[t, k], k in order.
+int yalm_moe_route(const void* h, const void* w_router, int dtype, int* ids, float* wts, int T, int D, int E, int top,
+                   int renorm, hipStream_t stream);
+int yalm_moe_pair_gate_up(const void* h, const void* w_gate, const void* w_up, const int* ids, float limit, float alpha,
+                          void* mid, int T, int top, int D, int F, int E, int dtype, hipStream_t stream);
+int yalm_moe_pair_down(const void* mid, const void* w_down, const int* ids, const float* wts, float* out, int T, int top,
+                       int D, int F, int E, int dtype, int accumulate, hipStream_t stream);
+
 // Yardsticks for the measurement (probes.hip): a kernel that only reads `bytes` bytes once with `workgroups`
 // workgroups (out: 1,024 words of scratch), and a loop of matrix-core instructions on registers (shape 32:
 // v_mfma_f32_32x32x16_bf16, 16: v_mfma_f32_16x16x32_bf16; *flops, host memory, receives the launch's operations).

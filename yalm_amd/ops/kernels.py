@@ -719,6 +719,134 @@ def attn_sink_mix(q, out, lse, sink_k, sink_v, tok_seq, tok_pos, seq_slot, cos_s
     return out
 
 
+# ---------------------------------------------------------------------------------------------------------------
+# layers that norm a sublayer's output; PolyNorm
+def cast(x, out):
+    """out = x (float32) in out's dtype, element by element."""
+    n = x.numel()
+    if out.numel() != n:
+        raise ValueError("cast: %d elements into %d" % (n, out.numel()))
+    library.check(library.lib().yalm_cast(_need(x, "x", torch.float32), _need(out, "out"), n, dtype_code(out.dtype),
+                                          _stream()), "cast")
+    return out
+
+
+def norm_add(y, weight, eps, x, h_out=None):
+    """x += y * rsqrt(mean(y^2) + eps) * weight, row by row (x, y float32 [R, D]); h_out (optional, [R, D] in the
+    compute dtype) receives the new x: the input of the sublayer that follows."""
+    R, D = y.shape
+    p_h, h_code = None, 0
+    if h_out is not None:
+        p_h, h_code = _need(h_out, "h_out", None, (R, D)), dtype_code(h_out.dtype)
+    library.check(library.lib().yalm_norm_add(
+        _need(y, "y", torch.float32, (R, D)), _need(weight, "weight", None, (D,)), dtype_code(weight.dtype), float(eps),
+        _need(x, "x", torch.float32, (R, D)), p_h, h_code, R, D, _stream()), "norm_add")
+    return x
+
+
+def polynorm(z, coef, eps, out):
+    """out[r] = a N(z[r]) + b N(z[r]^2) + c N(z[r]^3) + e, powers element by element, N(v) = v / sqrt(mean(v^2) + eps);
+    z float32 [R, F], coef float32 [4] = (a, b, c, e) on the device, out [R, F] in the compute dtype."""
+    R, F = z.shape
+    library.check(library.lib().yalm_polynorm(
+        _need(z, "z", torch.float32, (R, F)), _need(coef, "coef", torch.float32, (4,)), float(eps),
+        _need(out, "out", None, (R, F)), dtype_code(out.dtype), R, F, _stream()), "polynorm")
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# latent attention
+HEAD_MATMUL_MAX_K = 512
+
+
+def head_matmul(src, src_head, src_off, wt, out, out_head, out_off, scale=1.0, gate=None):
+    """For every row t and head h: out[t, h * out_head + out_off + n] = scale * sum_k src[t, h * src_head + src_off + k]
+    * wt[h, k, n], times sigmoid(gate[t, h * N + n]) if gate (float32 [T, >= H * N]) is given.  src and out are
+    2-D, their rows may be wider than the heads they hold; wt [H, K, N].  Types (src, wt, out): all float32;
+    float32, bfloat16, float32; all bfloat16."""
+    H, K, N = wt.shape
+    T = src.shape[0]
+    if K > HEAD_MATMUL_MAX_K:
+        raise ValueError("head_matmul: %d inner elements a head, at most %d" % (K, HEAD_MATMUL_MAX_K))
+    if src_off + K > src_head or out_off + N > out_head or H * src_head > src.shape[1] or H * out_head > out.shape[1]:
+        raise ValueError("head_matmul: %d heads of %d (+%d) -> %d (+%d) do not fit rows of %d and %d"
+                         % (H, K, src_off, N, out_off, src.shape[1], out.shape[1]))
+    p_g, g_row = None, 0
+    if gate is not None:
+        g_row = gate.stride(0)
+        if gate.dim() != 2 or gate.shape[0] != T or gate.shape[1] < H * N or gate.stride(1) != 1 \
+                or gate.dtype != torch.float32 or not gate.is_cuda:
+            raise ValueError("head_matmul: gate must be float32 [T, >= heads * N] with unit column stride on the GPU")
+        p_g = gate.data_ptr()
+    library.check(library.lib().yalm_head_matmul(
+        _need(src, "src", None, (T, None)), dtype_code(src.dtype), src.shape[1], src_head, src_off,
+        _need(wt, "wt"), dtype_code(wt.dtype), _need(out, "out", None, (T, None)), dtype_code(out.dtype), out.shape[1],
+        out_head, out_off, float(scale), p_g, g_row, T, H, K, N, _stream()), "head_matmul")
+    return out
+
+
+def latent_pack(proj, q_head, q_rot_off, kv_off, norm_w, eps, q_scale, out, n_heads, rot, rank, padded, has_kv):
+    """Fills out float32 [T, (n_heads + 2) * padded], the rows that rope_kv_write reads as n_heads query heads and
+    one KV head of size `padded`, each [rot | rank | zeros]: the rotated parts of the queries from proj (float32
+    [T, *]; head h at column h * q_head + q_rot_off) times q_scale, zeros in the padding, and with has_kv the key
+    [proj[kv_off + rank:][:rot] | c | 0] and the value [0 | c | 0], c the RMS norm (weights norm_w, eps) of
+    proj[kv_off:][:rank].  The queries' rank places are left for head_matmul."""
+    T = proj.shape[0]
+    p_n, n_code = None, 0
+    if has_kv:
+        p_n, n_code = _need(norm_w, "norm_w", None, (rank,)), dtype_code(norm_w.dtype)
+    library.check(library.lib().yalm_latent_pack(
+        _need(proj, "proj", torch.float32, (T, None)), proj.shape[1], q_head, q_rot_off, kv_off if has_kv else 0, p_n,
+        n_code, float(eps), float(q_scale), _need(out, "out", torch.float32, (T, (n_heads + 2) * padded)), T, n_heads,
+        rot, rank, padded, 1 if has_kv else 0, _stream()), "latent_pack")
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# mixture of experts
+MOE_MAX_EXPERTS = 1024
+
+
+def moe_route(h, w_router, ids, wts, renormalize=False):
+    """ids, wts [T, top]: the top experts of every row of h [T, D] by softmax(w_router h) over all experts
+    (float32 arithmetic, the lowest index on ties) and those scores (renormalize: divided by their sum)."""
+    T, D = h.shape
+    E = w_router.shape[0]
+    top = ids.shape[1]
+    if not 0 < top <= min(E, 64) or E > MOE_MAX_EXPERTS:
+        raise ValueError("moe_route: %d of %d experts is not offered (at most 64 of %d)" % (top, E, MOE_MAX_EXPERTS))
+    library.check(library.lib().yalm_moe_route(
+        _need(h, "h", None, (T, D)), _need(w_router, "w_router", h.dtype, (E, D)), dtype_code(h.dtype),
+        _need(ids, "ids", torch.int32, (T, top)), _need(wts, "wts", torch.float32, (T, top)), T, D, E, top,
+        1 if renormalize else 0, _stream()), "moe_route")
+
+
+def moe_pair_gate_up(h, w_gate, w_up, ids, limit, alpha, mid):
+    """mid[t * top + k] = g sigmoid(alpha g) (u + 1), g = min(w_gate[e] h[t], limit), u = clamp(w_up[e] h[t], +-limit)
+    for e = ids[t, k] (limit <= 0: unclamped); w_gate, w_up [E, F, D]."""
+    T, D = h.shape
+    E, F, _ = w_gate.shape
+    top = ids.shape[1]
+    dt = h.dtype
+    library.check(library.lib().yalm_moe_pair_gate_up(
+        _need(h, "h", dt, (T, D)), _need(w_gate, "w_gate", dt, (E, F, D)), _need(w_up, "w_up", dt, (E, F, D)),
+        _need(ids, "ids", torch.int32, (T, top)), float(limit), float(alpha), _need(mid, "mid", dt, (T * top, F)),
+        T, top, D, F, E, dtype_code(dt), _stream()), "moe_pair_gate_up")
+    return mid
+
+
+def moe_pair_down(mid, w_down, ids, wts, out, accumulate=False):
+    """out float32 [T, D] = (accumulate: out +) sum over k, in order, of wts[t, k] * w_down[ids[t, k]] mid[t * top + k]; w_down [E, D, F]."""
+    E, D, F = w_down.shape
+    T, top = ids.shape
+    dt = mid.dtype
+    library.check(library.lib().yalm_moe_pair_down(
+        _need(mid, "mid", dt, (T * top, F)), _need(w_down, "w_down", dt, (E, D, F)),
+        _need(ids, "ids", torch.int32, (T, top)), _need(wts, "wts", torch.float32, (T, top)),
+        _need(out, "out", torch.float32, (T, D)), T, top, D, F, E, dtype_code(dt), 1 if accumulate else 0, _stream()), "moe_pair_down")
+    return out
+
+
 def argmax(logits, out):
     R, V = logits.shape
     library.check(library.lib().yalm_argmax(_need(logits, "logits", torch.float32), _need(out, "out", torch.int32, (R,)),

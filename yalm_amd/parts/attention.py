@@ -48,6 +48,25 @@ def kv_tiles(n_tok):
 kv_tiles.name = "kv_tiles"
 
 
+def decode_splits(n_heads, n_kv_heads, head_dim, B, max_pages, ragged=False):
+    """Into how many pieces a decode step's attention cuts every sequence, so that about TARGET_WORKGROUPS
+    workgroups run."""
+    mfma = head_dim in kernels.MFMA_HEAD_DIMS and not kernels.FORCE_SIMPLE
+    if mfma:         # a workgroup of 4 waves per (split, KV head and up to 16 of its query heads, sequence), a page per wave at a time
+        per = max(1, B * n_kv_heads * ((n_heads // n_kv_heads + 15) // 16))
+        quarters = max(1, min((max_pages + 3) // 4, 4))
+        if per > RESIDENT_WORKGROUPS:         # more than run at once: in quarters the last round is short
+            return quarters
+        even = max(1, min((max_pages + 3) // 4, TARGET_WORKGROUPS // per))
+        # Sequences of very unequal lengths.  Where the workgroups stand two to a compute unit anyway, one split and
+        # the rows in the order that pairs a long sequence with a short one; else splits of the longest sequence's
+        # split size (the kernel cuts them so), enough of them that the long sequences' work spreads over the chip.
+        if ragged and per <= TARGET_WORKGROUPS:
+            return max(even, quarters)
+        return even
+    return max(1, min(max_pages, TARGET_WORKGROUPS // max(1, B * n_heads)))
+
+
 @part("mixer", "gqa_attention")
 class GQAttention(Part):
     prompt_tables = (kv_tiles,)
@@ -122,20 +141,7 @@ class GQAttention(Part):
                       "of 16 to 128 in steps of 16, not %d): correct, several times slower" % self.head_dim, True
 
     def decode_splits(self, B, max_pages, ragged=False):
-        mfma = self.head_dim in kernels.MFMA_HEAD_DIMS and not kernels.FORCE_SIMPLE
-        if mfma:         # a workgroup of 4 waves per (split, KV head and up to 16 of its query heads, sequence), a page per wave at a time
-            per = max(1, B * self.n_kv_heads * ((self.n_heads // self.n_kv_heads + 15) // 16))
-            quarters = max(1, min((max_pages + 3) // 4, 4))
-            if per > RESIDENT_WORKGROUPS:         # more than run at once: in quarters the last round is short
-                return quarters
-            even = max(1, min((max_pages + 3) // 4, TARGET_WORKGROUPS // per))
-            # Sequences of very unequal lengths.  Where the workgroups stand two to a compute unit anyway, one split and
-            # the rows in the order that pairs a long sequence with a short one; else splits of the longest sequence's
-            # split size (the kernel cuts them so), enough of them that the long sequences' work spreads over the chip.
-            if ragged and per <= TARGET_WORKGROUPS:
-                return max(even, quarters)
-            return even
-        return max(1, min(max_pages, TARGET_WORKGROUPS // max(1, B * self.n_heads)))
+        return decode_splits(self.n_heads, self.n_kv_heads, self.head_dim, B, max_pages, ragged)
 
     def fuses_norm(self, norm, x, ctx):
         if not hasattr(norm, "fused") or self.head_dim % 16:

@@ -38,3 +38,61 @@ class PreNormResidualBlock(Part):
             h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
             self.feed_forward_norm.forward(x, h, ctx)
             self.feed_forward.forward(h, x, ctx)
+
+
+class StreamInput:
+    """What `first_norm()` of a block that reads the residual stream itself hands to the layer before it: the
+    place under which that layer may leave the stream in the compute dtype (ctx.normed[id(...)] = (h, None,
+    None)), so that no kernel runs only to convert it."""
+
+
+@part("block", "postnorm_residual")
+class PostNormResidualBlock(Part):
+    """x += norm(mixer(x)); x += norm(feed_forward(x)): the sublayers read the residual stream itself and
+    the norms act on their OUTPUTS.  Members: mixer, mixer_norm, and optionally feed_forward with
+    feed_forward_norm (a layer may have no feed-forward).  The sublayers offer forward_to(h, y, ...),
+    which writes their result to y instead of adding it to the stream; the norm's add_normed(y, x, h_out)
+    adds it normed and hands the new stream on in the compute dtype.  With float32 as the compute dtype the
+    sublayers read the stream's own memory."""
+
+    def __init__(self, layer_spec, dim, prefix=""):
+        super().__init__(None, dim, layer_spec.prefix)
+        p = layer_spec.prefix
+        self.mixer = build_part("mixer", layer_spec.mixer, dim, p)
+        self.mixer_norm = build_part("norm", layer_spec.mixer_norm, dim, p)
+        self.feed_forward = self.feed_forward_norm = None
+        if layer_spec.part("feed_forward") is not None:
+            self.feed_forward = build_part("feed_forward", layer_spec.feed_forward, dim, p)
+            self.feed_forward_norm = build_part("norm", layer_spec.feed_forward_norm, dim, p)
+        self.entry = StreamInput()
+
+    def children(self):
+        return [c for c in (self.mixer, self.mixer_norm, self.feed_forward, self.feed_forward_norm) if c is not None]
+
+    def first_norm(self):
+        return self.entry
+
+    def forward(self, x, ctx, line, writes_cache=True, next_norm=None):
+        import torch
+        from ..ops import kernels
+        T = x.shape[0]
+        same = ctx.act_dtype == torch.float32          # the sublayers read x itself
+        left = ctx.normed.pop(id(self.entry), None)
+        if same:
+            h = x
+        elif left is not None:
+            h = left[0]
+        else:
+            h = kernels.cast(x, ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype))
+        hand_on = None if same or not isinstance(next_norm, StreamInput) else ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype)
+        y = ctx.ws.get("block.y", (T, self.dim), torch.float32)
+        self.mixer.forward_to(h, y, ctx, line, writes_cache)
+        if self.feed_forward is None:
+            self.mixer_norm.add_normed(y, x, ctx, h_out=hand_on)
+        else:
+            h = x if same else ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype)
+            self.mixer_norm.add_normed(y, x, ctx, h_out=None if same else h)
+            self.feed_forward.forward_to(h, y, ctx)
+            self.feed_forward_norm.add_normed(y, x, ctx, h_out=hand_on)
+        if hand_on is not None:
+            ctx.normed[id(next_norm)] = (hand_on, None, None)

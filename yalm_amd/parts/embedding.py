@@ -12,13 +12,14 @@ class TokenEmbedding(Part):
     def __init__(self, spec, dim, prefix):
         super().__init__(spec, dim, prefix)
         self.vocab_size = int(spec.params["vocab_size"])
+        self.tensor = self.prefix + str(spec.params.get("tensor", "weight"))      # the table's name in a folder
         self.table = None
 
     def param_specs(self):
-        return [ParamSpec(self.prefix + "weight", (self.vocab_size, self.dim), init="embedding")]
+        return [ParamSpec(self.tensor, (self.vocab_size, self.dim), init="embedding")]
 
     def load(self, get, compute_dtype, device):
-        self.table = place(get(self.prefix + "weight"), compute_dtype, device)
+        self.table = place(get(self.tensor), compute_dtype, device)
 
     def weight_bytes(self):
         return self.dim * self.table.element_size()          # one row per token
@@ -35,6 +36,7 @@ class LMHead(Part):
         super().__init__(spec, dim, prefix)
         self.vocab_size = int(spec.params["vocab_size"])
         self.tied = bool(spec.params.get("tied", False))
+        self.tensor = self.prefix + str(spec.params.get("tensor", "weight"))
         self.embedding = embedding
         self.weight = None
         if self.tied and embedding is None:
@@ -43,10 +45,10 @@ class LMHead(Part):
     def param_specs(self):
         if self.tied:
             return []
-        return [ParamSpec(self.prefix + "weight", (self.vocab_size, self.dim), init="linear", fan_in=self.dim)]
+        return [ParamSpec(self.tensor, (self.vocab_size, self.dim), init="linear", fan_in=self.dim)]
 
     def load(self, get, compute_dtype, device):
-        self.weight = self.embedding.table if self.tied else place(get(self.prefix + "weight"), compute_dtype, device)
+        self.weight = self.embedding.table if self.tied else place(get(self.tensor), compute_dtype, device)
 
     def weight_bytes(self):
         return self.weight.numel() * self.weight.element_size()

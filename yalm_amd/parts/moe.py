@@ -1,0 +1,81 @@
+"""Mixture of experts: `n_experts` small gated feed-forwards, of which a token uses the `top` whose router
+scores are largest.
+
+Router: s = softmax(W_router h) over all experts, in float32; the chosen experts' weights are their scores
+(`renormalize`: divided by their sum).  Expert: g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit),
+out = W_down (g sigmoid(alpha g) (u + 1)) (limit 0: no clamping).  The part's result is the weighted sum over
+a token's chosen experts, in the order of their scores.
+
+The experts' matrices are stacked at load ([E, F, D], [E, F, D], [E, D, F]); routing happens on the device
+(nothing of it reaches the host, so a decode step stays a captured graph), and every (token, choice) pair is
+served from its expert's weights."""
+import torch
+
+from ..ops import kernels
+from ..weights.loader import ParamSpec, place
+from .base import Part, part
+
+
+@part("feed_forward", "moe")
+class MixtureOfExperts(Part):
+    def __init__(self, spec, dim, prefix):
+        super().__init__(spec, dim, prefix)
+        p = spec.params
+        self.hidden = int(p["hidden"])
+        self.n_experts = int(p["n_experts"])
+        self.top = int(p["top"])
+        self.limit = float(p.get("limit", 0.0) or 0.0)
+        self.alpha = float(p.get("alpha", 1.0))
+        self.renormalize = bool(p.get("renormalize", False))
+        self.expert_prefix = str(p.get("expert_prefix", "experts.%d."))
+        self.names = {"router": "router", "gate": "gate", "up": "up", "down": "down"}
+        self.names.update(p.get("tensors") or {})
+        if not 0 < self.top <= self.n_experts or self.top > 64 or self.n_experts > kernels.MOE_MAX_EXPERTS:
+            raise ValueError("mixture of experts: %d of %d experts is not offered (at most 64 of %d)"
+                             % (self.top, self.n_experts, kernels.MOE_MAX_EXPERTS))
+        self.w_router = self.w_gate = self.w_up = self.w_down = None
+
+    def _expert(self, e, key):
+        return self.prefix + (self.expert_prefix % e) + self.names[key]
+
+    def param_specs(self):
+        D, F = self.dim, self.hidden
+        out = [ParamSpec(self.prefix + self.names["router"], (self.n_experts, D), fan_in=D)]
+        for e in range(self.n_experts):
+            out += [ParamSpec(self._expert(e, "gate"), (F, D), fan_in=D), ParamSpec(self._expert(e, "up"), (F, D), fan_in=D),
+                    ParamSpec(self._expert(e, "down"), (D, F), fan_in=F)]
+        return out
+
+    def load(self, get, compute_dtype, device):
+        E = self.n_experts
+        self.w_router = place(get(self.prefix + self.names["router"]), compute_dtype, device)
+        self.w_gate = place(torch.stack([get(self._expert(e, "gate")) for e in range(E)]), compute_dtype, device)
+        self.w_up = place(torch.stack([get(self._expert(e, "up")) for e in range(E)]), compute_dtype, device)
+        self.w_down = place(torch.stack([get(self._expert(e, "down")) for e in range(E)]), compute_dtype, device)
+
+    def weight_bytes(self):
+        """What a token's step reads: the router and `top` experts."""
+        item = self.w_down.element_size()
+        return (self.n_experts * self.dim + self.top * 3 * self.hidden * self.dim) * item
+
+    def row_elements(self):
+        return self.top * self.hidden
+
+    def _run(self, h, out, ctx, accumulate):
+        T = h.shape[0]
+        ws = ctx.ws
+        ids = ws.get("moe.ids", (T, self.top), torch.int32)
+        wts = ws.get("moe.weights", (T, self.top), torch.float32)
+        kernels.moe_route(h, self.w_router, ids, wts, self.renormalize)
+        mid = ws.get("moe.hidden", (T * self.top, self.hidden), h.dtype)
+        kernels.moe_pair_gate_up(h, self.w_gate, self.w_up, ids, self.limit, self.alpha, mid)
+        kernels.moe_pair_down(mid, self.w_down, ids, wts, out, accumulate)
+        return out
+
+    def forward(self, h, x, ctx):
+        """Adds the result to x."""
+        return self._run(h, x, ctx, True)
+
+    def forward_to(self, h, y, ctx):
+        """Writes the result to y (float32 [T, dim])."""
+        return self._run(h, y, ctx, False)

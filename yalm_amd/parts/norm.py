@@ -1,5 +1,7 @@
 """RMSNorm: out = x * rsqrt(mean(x^2) + eps) * weight, sums in float32
-(src/infer.cpp:136-146, src/infer.cu:525-539)."""
+(src/infer.cpp:136-146, src/infer.cu:525-539).  The parameter `tensor` names the weight behind the
+part's prefix (default "weight").  `add_normed` is the norm of a layer that norms a sublayer's OUTPUT:
+x += norm(y)."""
 import torch
 
 from ..ops import kernels
@@ -12,13 +14,14 @@ class RMSNorm(Part):
     def __init__(self, spec, dim, prefix):
         super().__init__(spec, dim, prefix)
         self.eps = float(spec.params["eps"])
+        self.tensor = self.prefix + str(spec.params.get("tensor", "weight"))
         self.weight = None
 
     def param_specs(self):
-        return [ParamSpec(self.prefix + "weight", (self.dim,), init="norm")]
+        return [ParamSpec(self.tensor, (self.dim,), init="norm")]
 
     def load(self, get, compute_dtype, device):
-        self.weight = place(get(self.prefix + "weight"), compute_dtype, device)
+        self.weight = place(get(self.tensor), compute_dtype, device)
         self.weight_f32 = self.weight if self.weight.dtype == torch.float32 else self.weight.float()
 
     def weight_bytes(self):
@@ -30,3 +33,7 @@ class RMSNorm(Part):
 
     def forward(self, x, out, ctx, row_index=None):
         return kernels.rmsnorm(x, self.weight, out, self.eps, row_index)
+
+    def add_normed(self, y, x, ctx, h_out=None):
+        """x += norm(y) (both float32 [T, dim]); h_out, if given, receives the new x in the compute dtype."""
+        return kernels.norm_add(y, self.weight, self.eps, x, h_out)

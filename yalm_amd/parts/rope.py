@@ -5,6 +5,11 @@ f_p = theta^(-2p / rotary_dim), optionally rescaled the llama3 way (not in the
 reference): with wavelength lam = 2 pi / f and L the original context length,
 lam < L/high -> f; lam > L/low -> f/factor; between, the linear blend
 (1-s) f/factor + s f with s = (L/lam - low) / (high - low).
+Or the YaRN way (`rope_type` "yarn": factor, original_max_position_embeddings L, beta_fast, beta_slow):
+with n(t) = rotary_dim ln(L / (2 pi t)) / (2 ln theta) the index of the pair that makes t turns within L,
+lo = max(floor(n(beta_fast)), 0), hi = min(ceil(n(beta_slow)), rotary_dim - 1) and the ramp r_p = clamp((p - lo) /
+max(hi - lo, 0.001), 0, 1), the frequency is (1 - r_p) f_p + r_p f_p / factor, and cos and sin are both multiplied
+by 0.1 ln(factor) + 1 (`table_magnitude`).
 
 A model folder keeps q/k projection rows in the half-split order (pair p with
 p + rotary_dim/2); `interleave_rows` re-orders them for adjacent pairs, as
@@ -22,6 +27,16 @@ def inverse_frequencies(head_dim, rotary_dim, theta, scaling=None):
     f = torch.pow(torch.tensor(float(theta), dtype=torch.float64), -2.0 * p / max(rotary_dim, 1))
     if scaling:
         kind = scaling.get("rope_type", scaling.get("type"))
+        if kind == "yarn":
+            factor, L = float(scaling["factor"]), float(scaling["original_max_position_embeddings"])
+
+            def pair_of(turns):
+                return rotary_dim * math.log(L / (2.0 * math.pi * turns)) / (2.0 * math.log(float(theta)))
+
+            lo = max(math.floor(pair_of(float(scaling["beta_fast"]))), 0)
+            hi = min(math.ceil(pair_of(float(scaling["beta_slow"]))), rotary_dim - 1)
+            ramp = torch.clamp((p - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+            return f / factor * ramp + f * (1.0 - ramp)
         if kind != "llama3":
             raise ValueError("rope scaling %r is not supported" % (kind,))
         factor = float(scaling["factor"])
@@ -32,6 +47,13 @@ def inverse_frequencies(head_dim, rotary_dim, theta, scaling=None):
         blend = (1.0 - s) * f / factor + s * f
         f = torch.where(lam < L / high, f, torch.where(lam > L / low, f / factor, blend))
     return f
+
+
+def table_magnitude(scaling=None):
+    """The factor on both cos and sin of the table (1 unless the scaling is YaRN's)."""
+    if scaling and scaling.get("rope_type", scaling.get("type")) == "yarn":
+        return 0.1 * math.log(float(scaling["factor"])) + 1.0
+    return 1.0
 
 
 def interleave_rows(w, n_heads, head_dim, rotary_dim):
@@ -66,7 +88,8 @@ class RotaryEncoding(Part):
             return
         f = inverse_frequencies(self.head_dim, self.rotary_dim, self.theta, self.scaling)
         ang = torch.arange(n_positions, dtype=torch.float64)[:, None] * f[None, :]
-        self.table = torch.stack([torch.cos(ang), torch.sin(ang)], dim=-1).to(torch.float32).contiguous().to(device)
+        mag = table_magnitude(self.scaling)
+        self.table = torch.stack([torch.cos(ang) * mag, torch.sin(ang) * mag], dim=-1).to(torch.float32).contiguous().to(device)
 
     @property
     def n_positions(self):
