@@ -137,6 +137,17 @@ def route(h, w, prefix, top):
     return chosen, weight
 
 
+def route_margin(h, w, prefix, top):
+    """How decided the router's choice is, per token: the gap between the last chosen and the first
+    unchosen logit, relative to the logits' root mean square (infinite if every expert is chosen).  A
+    computation in fewer bits may choose otherwise where this is small."""
+    z = h @ w[prefix + "router"].to(F64).T
+    if top >= z.shape[-1]:
+        return torch.full((h.shape[0],), float("inf"), dtype=F64)
+    best = torch.topk(z, top + 1, dim=-1).values
+    return (best[:, top - 1] - best[:, top]) / torch.sqrt((z * z).mean(dim=-1))
+
+
 def moe_ff(h, mlp, w, prefix):
     top, limit = int(mlp["router"]["top"]), float(mlp["expert"]["limit"])
     chosen, weight = route(h, w, prefix, top)
@@ -157,10 +168,11 @@ def feed_forward(h, mlp, w, prefix, eps):
 
 
 # ------------------------------------------------------------------------------------------ the model
-def forward(config, w, tokens, memory=None, start=0, layers_out=None):
+def forward(config, w, tokens, memory=None, start=0, layers_out=None, margins_out=None):
     """Logits [T, vocab] of one sequence's tokens at positions start.. .  memory: {layer: (c, k_rot)}
     of the positions before `start`, extended in place (pass {} and call again to go on token by
-    token).  layers_out: a list that receives the residual stream after every layer."""
+    token).  layers_out: a list that receives the residual stream after every layer; margins_out: a list that
+    receives route_margin [T] of every mixture-of-experts layer."""
     eps = float(config["norm"]["eps"])
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     T = tokens.shape[0]
@@ -181,6 +193,8 @@ def forward(config, w, tokens, memory=None, start=0, layers_out=None):
                                 memory=(c, k_rot, torch.arange(c.shape[0])), visible=visibility(mixer))
         x = x + rms_norm(y, w[p + "norm1"].to(F64), eps)
         if layer.get("mlp"):
+            if margins_out is not None and layer["mlp"]["kind"] == "moe":
+                margins_out.append(route_margin(x, w, p + "mlp.", int(layer["mlp"]["router"]["top"])))
             y = feed_forward(x, layer["mlp"], w, p + "mlp.", eps)
             x = x + rms_norm(y, w[p + "norm2"].to(F64), eps)
         if layers_out is not None:

@@ -84,7 +84,8 @@ __global__ __launch_bounds__(WAVE) void moe_route_kernel(const T* __restrict__ h
     total += best;
     __syncthreads();
   }
-  if (renorm && lane < top) wts[(size_t)t * top + lane] /= total;
+  if (renorm)
+    for (int k = lane; k < top; k += WAVE) wts[(size_t)t * top + k] /= total;
 }
 
 template <typename T>
@@ -134,7 +135,7 @@ __global__ __launch_bounds__(PAIR_WAVES * WAVE) void moe_pair_down_kernel(const 
 extern "C" int yalm_moe_route(const void* h, const void* w_router, int dtype, int* ids, float* wts, int T, int D, int E,
                               int top, int renorm, hipStream_t stream) {
   if (T <= 0) return YALM_OK;
-  if (D <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > E || top > WAVE) return YALM_ERR_ARG;
+  if (D <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > E) return YALM_ERR_ARG;
   if (dtype == YALM_BF16)
     moe_route_kernel<bf16><<<T, WAVE, 0, stream>>>((const bf16*)h, (const bf16*)w_router, ids, wts, D, E, top, renorm);
   else if (dtype == YALM_F32)

@@ -813,8 +813,8 @@ def moe_route(h, w_router, ids, wts, renormalize=False):
     T, D = h.shape
     E = w_router.shape[0]
     top = ids.shape[1]
-    if not 0 < top <= min(E, 64) or E > MOE_MAX_EXPERTS:
-        raise ValueError("moe_route: %d of %d experts is not offered (at most 64 of %d)" % (top, E, MOE_MAX_EXPERTS))
+    if not 0 < top <= E or E > MOE_MAX_EXPERTS:
+        raise ValueError("moe_route: %d of %d experts is not offered (at most %d experts)" % (top, E, MOE_MAX_EXPERTS))
     library.check(library.lib().yalm_moe_route(
         _need(h, "h", None, (T, D)), _need(w_router, "w_router", h.dtype, (E, D)), dtype_code(h.dtype),
         _need(ids, "ids", torch.int32, (T, top)), _need(wts, "wts", torch.float32, (T, top)), T, D, E, top,

@@ -30,8 +30,8 @@ class MixtureOfExperts(Part):
         self.expert_prefix = str(p.get("expert_prefix", "experts.%d."))
         self.names = {"router": "router", "gate": "gate", "up": "up", "down": "down"}
         self.names.update(p.get("tensors") or {})
-        if not 0 < self.top <= self.n_experts or self.top > 64 or self.n_experts > kernels.MOE_MAX_EXPERTS:
-            raise ValueError("mixture of experts: %d of %d experts is not offered (at most 64 of %d)"
+        if not 0 < self.top <= self.n_experts or self.n_experts > kernels.MOE_MAX_EXPERTS:
+            raise ValueError("mixture of experts: %d of %d experts is not offered (at most %d experts)"
                              % (self.top, self.n_experts, kernels.MOE_MAX_EXPERTS))
         self.w_router = self.w_gate = self.w_up = self.w_down = None
 
