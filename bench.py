@@ -8,11 +8,18 @@ shape with its window of 4,096 positions and prompts of 6,000 tokens).
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--dtype bf16|fp32] [--shape NAME]
                     [--prompt-len N] [--prefill-len N] [--batch B] [--points B,B] [--no-prefill]
                     [--kernels] [--ragged] [--sweep]
+    python bench.py --design situlorn [--sizes 2048,4096] [--kernels] [--steps K] [--warmup W]
 
 --kernels adds the time of every kernel of a decode step and of a prompt step, each taken alone at the
 shape's sizes (src/test.cpp:340-405 times single kernels so), with its rate against the peak;
 --ragged adds generate() over 64 requests of unequal lengths beside the same batch at equal lengths;
 --sweep adds the shape's whole workload end to end (src/main.cpp:104-147 times a whole run).
+
+--design situlorn measures another model design beside the closest one the library has: four layers of the
+Situlorn design (latent attention with and without a window, one layer on another's keys, dense PolyNorm and
+mixture-of-experts feed-forwards) and four Llama layers of the same width and about the same weights, each a
+prompt of --prefill-len tokens and decode steps at --batch; with --kernels every kernel of both alone.  The default
+workload and its line stay as they are.
 
 A step is one decode step as generation does it: the step function for a batch
 of sequences (one token each, from the cache), greedy sampling on the device
@@ -102,7 +109,8 @@ def measured_peaks(torch, dtype):
 
 KERNEL_FACES = ("embed", "rmsnorm", "gemm", "gemm_norm", "gemm_norm_qkv_rope", "gemm_add_norm", "gemm_add_emit", "gemm_partial",
                 "gemm_chain", "gemm_chain_qkv_rope", "rope_kv_write", "rope_kv_write_tiles", "attn_prefill",
-                "attn_decode", "sink_store", "attn_sink_mix", "argmax")
+                "attn_decode", "sink_store", "attn_sink_mix", "argmax", "cast", "norm_add", "polynorm", "head_matmul",
+                "latent_pack", "moe_route", "moe_pair_gate_up", "moe_pair_down", "moe_grouped")
 
 
 def record_kernel_calls(run):
@@ -165,6 +173,31 @@ def kernel_cost(name, a, kw, kv_tokens, torch):
         return "embed %d" % a[1].shape[0], 2 * nbytes(a[2]), 0.0
     if name == "argmax":
         return "argmax %dx%d" % tuple(a[0].shape), nbytes(a[0]), 0.0
+    if name == "head_matmul":
+        src, wt, out = a[0], a[3], a[4]
+        H, K, N = wt.shape
+        T = src.shape[0]
+        return "head_matmul %dx%dx%dx%d" % (T, H, K, N), nbytes(wt) + T * H * (K * src.element_size() + N * out.element_size()), \
+            2.0 * T * H * K * N
+    if name == "latent_pack":
+        return "latent_pack %d tokens" % a[0].shape[0], nbytes(a[7]), 0.0
+    if name == "norm_add":
+        return "norm_add %dx%d" % tuple(a[0].shape), 3 * nbytes(a[0]), 0.0
+    if name == "polynorm":
+        return "polynorm %dx%d" % tuple(a[0].shape), nbytes(a[0], a[3]), 0.0
+    if name == "cast":
+        return "cast %d" % a[0].numel(), nbytes(a[0], a[1]), 0.0
+    if name == "moe_route":
+        return "moe_route %d tokens" % a[0].shape[0], nbytes(a[0], a[1]), 2.0 * a[0].shape[0] * a[1].numel()
+    if name in ("moe_pair_gate_up", "moe_pair_down", "moe_grouped"):
+        h, w = a[0], a[1]
+        ids = a[4] if name == "moe_grouped" else (a[3] if name == "moe_pair_gate_up" else a[2])
+        pairs = ids.numel()
+        E = w.shape[0]
+        per_expert = w[0].numel() * w.element_size()
+        mats = {"moe_pair_gate_up": 2, "moe_pair_down": 1, "moe_grouped": 3}[name]
+        # every expert that some pair chose is read once (at most all of them)
+        return "%s %d pairs" % (name, pairs), min(pairs, E) * mats * per_expert + nbytes(h), 2.0 * pairs * mats * w[0].numel()
     return name, nbytes(*a), 0.0
 
 
@@ -224,6 +257,113 @@ def mean_of(values):
     return int(sum(values) / len(values))
 
 
+def situlorn_config(width, n_layers=4):
+    """Layers of the Situlorn design at a real model's sizes.  The latent head (rotated part + latent vector) is
+    128 wide, the widest the matrix-core attention kernels take."""
+    heads = width // 128
+    rot = {"base": 10000.0, "dims": 32}
+    yarn = dict(rot, scaling={"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0})
+    full = {"heads": heads, "dim": 96, "rot_dim": 32, "vdim": 128, "kv_rank": 96, "scale": 128 ** -0.5, "rot": rot}
+    windowed = dict(full, rot=yarn, mask={"size": 1024})
+    dense = {"kind": "dense", "ff": width * 21 // 4}               # two matrices: as many weights as a gated one of 3.5 width
+    moe = {"kind": "moe", "expert": {"ff": width // 2, "limit": 7.0}, "router": {"experts": 32, "top": 4}}
+    pattern = [{"type": "latent_attention", "mixer": full, "mlp": dense},
+               {"type": "latent_attention", "mixer": dict(full, kv_from=0), "mlp": moe},
+               {"type": "latent_attention_2", "mixer": windowed, "mlp": dense},
+               {"type": "latent_attention_2", "mixer": windowed, "mlp": moe}]
+    return {"architecture": "Situlorn", "vocab": 32000, "width": width, "norm": {"eps": 1e-5},
+            "layers": [pattern[i % 4] for i in range(n_layers)]}
+
+
+def llama_config(width, n_layers=4):
+    return {"architectures": ["LlamaForCausalLM"], "hidden_size": width, "intermediate_size": width * 7 // 2,
+            "num_hidden_layers": n_layers, "num_attention_heads": width // 128, "num_key_value_heads": width // 512,
+            "head_dim": 128, "vocab_size": 32000, "max_position_embeddings": 32768, "rope_theta": 10000.0,
+            "rms_norm_eps": 1e-5, "hidden_act": "silu", "tie_word_embeddings": False}
+
+
+def bench_design(args):
+    """Prompt and decode steps of the Situlorn design beside Llama layers of equal width, with every kernel alone on
+    request.  One JSON line."""
+    import torch
+    from yalm_amd import Engine, Model, Sampler
+    dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
+    B, T, PROMPT = args.batch, args.prefill_len, args.prompt_len or 2048
+    gen = torch.Generator().manual_seed(1)
+    sampler = Sampler(0)
+    out = {}
+    for width in [int(w) for w in args.sizes.split(",") if w]:
+        for design, cfg in (("situlorn", situlorn_config(width)), ("llama", llama_config(width))):
+            model = Model.random(cfg, seed=0, dtype=dtype, device="cuda:0")
+            V = model.vocab_size
+            engine = Engine(model, max_tokens=B * (PROMPT + args.steps + args.warmup + 128) + T + 64, max_batch=B)
+            engine.warmup([B], min_len=PROMPT + 1, max_len=PROMPT + args.steps + args.warmup + 2)
+            prompt = torch.randint(0, V, (T,), generator=gen).tolist()
+            times = []
+            for _ in range(3):
+                slots = engine.start(1)
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                sampler.sample(engine.step(slots, [prompt]), 0.0, [0], [0])
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t)
+                engine.release(slots)
+            prefill_s = min(times[1:])
+            prompts = [torch.randint(0, V, (PROMPT,), generator=gen).tolist() for _ in range(B)]
+            slots, ids = engine.start(B), list(range(B))
+            tokens = []
+            for i in range(0, B, 4):
+                tokens += sampler.sample(engine.step(slots[i:i + 4], prompts[i:i + 4]), 0.0, ids[i:i + 4], [0] * len(slots[i:i + 4]))
+            drawn = sampler.draw(engine.step(slots, [[t] for t in tokens]), 0.0, ids, [0] * B)
+
+            def advance(n, drawn):
+                for _ in range(n):
+                    ahead = sampler.draw(engine.step_from(slots, drawn.tokens), 0.0, ids, [0] * B)
+                    drawn.tolist()
+                    drawn = ahead
+                return drawn
+            drawn = advance(args.warmup, drawn)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            advance(args.steps, drawn)
+            torch.cuda.synchronize()
+            step_s = (time.perf_counter() - t) / args.steps
+            ctx_len = engine.length(slots[0]) - args.steps / 2.0
+            kv = sum(g.bytes_per_token() * (min(ctx_len, g.window) if g.window else ctx_len) for g in engine.cache.kv_groups) * B
+            step_bytes = model.weight_bytes() + kv
+            r = {"prefill_tokens": T, "prefill_ms": round(prefill_s * 1e3, 3), "prefill_tok_s": round(T / prefill_s, 1),
+                 "decode_batch": B, "decode_context": int(ctx_len), "decode_ms_per_step": round(step_s * 1e3, 4),
+                 "decode_tok_s": round(B / step_s, 1), "decode_step_MB": round(step_bytes / 1e6, 1),
+                 "decode_hbm_frac": round(step_bytes / step_s / HBM_PEAK, 4), "weights_MB": round(model.weight_bytes() / 1e6, 1)}
+            sys.stderr.write("[bench] width %d %-8s %s\n" % (width, design, r))
+            if args.kernels:
+                engine.use_graphs = False
+                calls = record_kernel_calls(lambda: sampler.draw(engine.step(slots, [[1]] * B), 0.0, ids, [0] * B))
+                torch.cuda.synchronize()
+                per = time_kernel_groups(calls, int(B * ctx_len), torch, args.dtype)
+                r["kernels_decode"] = dict(per, sum_us=round(sum(k["us"] * k["calls"] for k in per.values()), 1))
+                for label, k in per.items():
+                    sys.stderr.write("[bench]   decode  %-46s x%-3d %8.2f us %8.1f GB/s %8.2f TFLOP/s  %.3f of %s\n"
+                                     % (label, k["calls"], k["us"], k["GB/s"], k["TFLOP/s"], k["frac"], k["bound"]))
+                engine.release(slots)
+                slots = engine.start(1)
+                calls = record_kernel_calls(lambda: sampler.draw(engine.step(slots, [prompt]), 0.0, [0], [0]))
+                torch.cuda.synchronize()
+                per = time_kernel_groups(calls, 0, torch, args.dtype)
+                r["kernels_prefill"] = dict(per, sum_us=round(sum(k["us"] * k["calls"] for k in per.values()), 1))
+                for label, k in per.items():
+                    sys.stderr.write("[bench]   prefill %-46s x%-3d %8.2f us %8.1f GB/s %8.2f TFLOP/s  %.3f of %s\n"
+                                     % (label, k["calls"], k["us"], k["GB/s"], k["TFLOP/s"], k["frac"], k["bound"]))
+            engine.release(slots)
+            out["%s_%d" % (design, width)] = r
+            del engine, model
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": "prompt and decode steps of 4 Situlorn layers beside 4 Llama layers of equal width",
+                      "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype,
+                      "data": "synthetic: seeded random weights and token ids", "sizes": out}), flush=True)
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -252,10 +392,16 @@ def main():
     ap.add_argument("--context", type=int, default=0,
                     help="the reference's -T: past this many positions two attention sinks and the last "
                          "<context> - 2 positions are attended to (0: the shape's own window, if any)")
+    ap.add_argument("--design", default="", choices=["", "situlorn"],
+                    help="measure layers of this design beside Llama layers of equal width instead of the default workload")
+    ap.add_argument("--sizes", default="2048,4096", help="widths for --design")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this library runs on one GPU; --gpus %d is not measured" % args.gpus, flush=True)
         return 2
+
+    if args.design:
+        return bench_design(args)
 
     import torch
     from yalm_amd import Engine, Model, Sampler

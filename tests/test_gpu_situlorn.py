@@ -153,6 +153,44 @@ def test_router_and_experts(dtype, T, D, E, top):
         assert torch.allclose(out.cpu().to(F64), 2 * want, rtol=tol, atol=2 * tol * max(1.0, float(want.abs().max())))
 
 
+@pytest.mark.parametrize("T,D,E,top,F", [(3, 16, 2, 1, 8), (130, 80, 6, 2, 48), (300, 96, 16, 3, 40), (64, 64, 5, 5, 72),
+                                         (257, 200, 40, 4, 24)])
+def test_grouped_experts_equal_the_pair_kernels(T, D, E, top, F):
+    """The grouped products of a prompt step against the (token, choice) kernels on the same operands: a
+    matter of summation order only.  Experts without a token, experts with more than a tile of them."""
+    from yalm_amd.ops import kernels
+    dt = torch.bfloat16
+    h = randn(T, D, seed=20).to(dt).to(DEV)
+    router = randn(E, D, seed=21, scale=D ** -0.5)
+    router[E // 2] = 0.0
+    router[E // 2, 0] = -100.0 if E > 2 else 0.0                # an expert that (almost) nobody chooses
+    wg = randn(E, F, D, seed=22, scale=2.0 * D ** -0.5).to(dt).to(DEV)
+    wu = randn(E, F, D, seed=23, scale=2.0 * D ** -0.5).to(dt).to(DEV)
+    wd = randn(E, D, F, seed=24, scale=F ** -0.5).to(dt).to(DEV)
+    ids = torch.zeros(T, top, dtype=torch.int32, device=DEV)
+    wts = torch.zeros(T, top, dtype=torch.float32, device=DEV)
+    kernels.moe_route(h, router.to(dt).to(DEV), ids, wts)
+    mid = torch.zeros(T * top, F, dtype=dt, device=DEV)
+    want = torch.zeros(T, D, device=DEV)
+    kernels.moe_pair_gate_up(h, wg, wu, ids, 1.2, 1.702, mid)
+    kernels.moe_pair_down(mid, wd, ids, wts, want)
+    bufs = {}
+
+    def scratch(name, shape, dtype):
+        bufs[name] = torch.full(shape, float("nan") if dtype.is_floating_point else -7, dtype=dtype, device=DEV)
+        return bufs[name]
+    got = torch.full((T, D), 3.0, device=DEV)
+    kernels.moe_grouped(h, wg, wu, wd, ids, wts, 1.2, 1.702, scratch, got)
+    scale = max(1.0, float(want.abs().max()))
+    assert torch.isfinite(got).all()
+    assert float((got - want).abs().max()) <= 2e-2 * scale
+    rows = bufs["moe.pair_of_row"].cpu()
+    assert sorted(rows[rows >= 0].tolist()) == list(range(T * top))           # every pair has one row
+    assert torch.equal(rows[bufs["moe.row_of_pair"].cpu().long()], torch.arange(T * top, dtype=torch.int32))
+    kernels.moe_grouped(h, wg, wu, wd, ids, wts, 1.2, 1.702, scratch, got, accumulate=True)
+    assert float((got - 2 * want).abs().max()) <= 4e-2 * scale
+
+
 def test_router_takes_the_lowest_index_among_equals():
     from yalm_amd.ops import kernels
     h = torch.ones(2, 8, device=DEV)

@@ -130,6 +130,196 @@ __global__ __launch_bounds__(PAIR_WAVES * WAVE) void moe_pair_down_kernel(const 
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// Many tokens (a step of whole prompts): the pairs are grouped by expert, every expert's rows padded to whole
+// tiles of GR_TM rows, and one launch multiplies all tiles on the matrix cores, each with its expert's weights.
+//
+// moe_group_kernel (one workgroup): counts the pairs of every expert, lays the experts' row blocks one behind
+// the other (each a multiple of GR_TM rows), and writes pair_of_row[row] (-1: padding), row_of_pair[pair] and
+// tile_expert[tile] (-1: behind the last used tile).  The order of an expert's rows among themselves is not
+// fixed, and no result depends on it: a row of a product depends on that row alone.
+// ---------------------------------------------------------------------------
+constexpr int GR_TM = 128, GR_TN = 128, GR_TK = 64, GR_ROW = GR_TK + 8, GR_THREADS = 256;
+constexpr int GROUP_THREADS = 1024;
+
+__global__ __launch_bounds__(GROUP_THREADS) void moe_group_kernel(const int* __restrict__ ids, int n_pairs, int E, int max_tiles,
+                                                                  int* __restrict__ pair_of_row, int* __restrict__ row_of_pair,
+                                                                  int* __restrict__ tile_expert) {
+  __shared__ int count[MOE_MAX_EXPERTS];
+  __shared__ int start[MOE_MAX_EXPERTS];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += GROUP_THREADS) count[e] = 0;
+  for (int r = tid; r < max_tiles * GR_TM; r += GROUP_THREADS) pair_of_row[r] = -1;
+  for (int t = tid; t < max_tiles; t += GROUP_THREADS) tile_expert[t] = -1;
+  __syncthreads();
+  for (int p = tid; p < n_pairs; p += GROUP_THREADS) {
+    const int e = ids[p];
+    if (e >= 0 && e < E) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int at = 0;
+    for (int e = 0; e < E; ++e) {
+      start[e] = at * GR_TM;
+      const int tiles = (count[e] + GR_TM - 1) / GR_TM;
+      for (int i = 0; i < tiles && at + i < max_tiles; ++i) tile_expert[at + i] = e;
+      at += tiles;
+      count[e] = 0;
+    }
+  }
+  __syncthreads();
+  for (int p = tid; p < n_pairs; p += GROUP_THREADS) {
+    const int e = ids[p];
+    if (e < 0 || e >= E) { row_of_pair[p] = -1; continue; }
+    const int row = start[e] + atomicAdd(&count[e], 1);
+    if (row < max_tiles * GR_TM) {
+      pair_of_row[row] = p;
+      row_of_pair[p] = row;
+    } else {
+      row_of_pair[p] = -1;
+    }
+  }
+}
+
+typedef __attribute__((ext_vector_type(8))) __bf16 gr_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float gr_f32x16;
+
+// A tile of GR_TM rows x GR_TN weight rows, 4 waves, each 32 rows x all weight rows (v_mfma_f32_32x32x16_bf16:
+// operand rows = lane % 32, 8 k a lane at k offset 8 * (lane / 32); C: column = lane % 32, rows 8 (r / 4) + 4
+// (lane / 32) + r % 4).  One LDS buffer, the next k tile waits in registers.
+// GATED: A rows are gathered (row -> pair -> token), the weight rows are 64 gate rows and the 64 up rows of the
+// same hidden columns, and the epilogue writes mid[row, f] = act(g, u).  Else: A = mid rows as they lie, the
+// weight rows are 128 rows of the expert's down matrix, and the epilogue stores float32 out[row, n].
+template <bool GATED>
+__global__ __launch_bounds__(GR_THREADS, 2) void moe_grouped_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W0,
+                                                                    const bf16* __restrict__ W1, const int* __restrict__ tile_expert,
+                                                                    const int* __restrict__ pair_of_row, int top, void* __restrict__ Cv,
+                                                                    int N, int K, float limit, float alpha) {
+  const int e = tile_expert[blockIdx.y];
+  if (e < 0) return;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16* As = reinterpret_cast<bf16*>(smem_raw);       // [GR_TM][GR_ROW]
+  bf16* Ws = As + GR_TM * GR_ROW;                      // [GR_TN][GR_ROW]
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int li = lane % 32, lh = lane / 32;
+  const int m0 = blockIdx.y * GR_TM;
+  const int n0 = blockIdx.x * (GATED ? GR_TN / 2 : GR_TN);      // first output column of the tile
+  constexpr int RPP = GR_THREADS / 8;                  // 32 rows a pass
+  constexpr int LA = GR_TM / RPP, LB = GR_TN / RPP;    // 4 chunks of 16 bytes a thread and operand
+  const int lrow = tid / 8, lk = (tid % 8) * 8;
+  const bf16* ap[LA];
+  const bf16* wp[LB];
+  bool aok[LA], wok[LB];
+#pragma unroll
+  for (int p = 0; p < LA; ++p) {
+    const int row = m0 + lrow + RPP * p;
+    if (GATED) {
+      const int pair = pair_of_row[row];
+      aok[p] = pair >= 0;
+      ap[p] = A + (size_t)(aok[p] ? pair / top : 0) * K + lk;
+    } else {
+      aok[p] = pair_of_row[row] >= 0;
+      ap[p] = A + (size_t)row * K + lk;
+    }
+  }
+#pragma unroll
+  for (int p = 0; p < LB; ++p) {
+    const int j = lrow + RPP * p;                      // row of the weight tile
+    int n;
+    const bf16* base;
+    if (GATED) {
+      n = n0 + (j % (GR_TN / 2));
+      base = j < GR_TN / 2 ? W0 : W1;
+    } else {
+      n = n0 + j;
+      base = W0;
+    }
+    wok[p] = n < N;
+    wp[p] = base + ((size_t)e * N + (wok[p] ? n : 0)) * K + lk;
+  }
+  gr_f32x16 acc[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[b][r] = 0.f;
+  const gr_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  gr_bf16x8 ra[LA], rw[LB];
+  const int nk = (K + GR_TK - 1) / GR_TK;
+  {
+    const bool kok = lk < K;
+#pragma unroll
+    for (int p = 0; p < LA; ++p) ra[p] = aok[p] && kok ? *reinterpret_cast<const gr_bf16x8*>(ap[p]) : zero;
+#pragma unroll
+    for (int p = 0; p < LB; ++p) rw[p] = wok[p] && kok ? *reinterpret_cast<const gr_bf16x8*>(wp[p]) : zero;
+  }
+  for (int kt = 0; kt < nk; ++kt) {
+#pragma unroll
+    for (int p = 0; p < LA; ++p) *reinterpret_cast<gr_bf16x8*>(&As[(lrow + RPP * p) * GR_ROW + lk]) = ra[p];
+#pragma unroll
+    for (int p = 0; p < LB; ++p) *reinterpret_cast<gr_bf16x8*>(&Ws[(lrow + RPP * p) * GR_ROW + lk]) = rw[p];
+    __syncthreads();
+    if (kt + 1 < nk) {
+      const bool kok = (kt + 1) * GR_TK + lk < K;
+#pragma unroll
+      for (int p = 0; p < LA; ++p)
+        ra[p] = aok[p] && kok ? *reinterpret_cast<const gr_bf16x8*>(ap[p] + (size_t)(kt + 1) * GR_TK) : zero;
+#pragma unroll
+      for (int p = 0; p < LB; ++p)
+        rw[p] = wok[p] && kok ? *reinterpret_cast<const gr_bf16x8*>(wp[p] + (size_t)(kt + 1) * GR_TK) : zero;
+    }
+#pragma unroll
+    for (int ks = 0; ks < GR_TK / 16; ++ks) {
+      const gr_bf16x8 fa = *reinterpret_cast<const gr_bf16x8*>(&As[(wave * 32 + li) * GR_ROW + ks * 16 + lh * 8]);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const gr_bf16x8 fw = *reinterpret_cast<const gr_bf16x8*>(&Ws[(b * 32 + li) * GR_ROW + ks * 16 + lh * 8]);
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fw, acc[b], 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int row = m0 + wave * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+    if (pair_of_row[row] < 0) continue;
+    if (GATED) {
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const int f = n0 + b * 32 + li;
+        if (f >= N) continue;
+        float g = acc[b][r], u = acc[b + 2][r];
+        if (limit > 0.f) {
+          g = fminf(g, limit);
+          u = fminf(fmaxf(u, -limit), limit);
+        }
+        ((bf16*)Cv)[(size_t)row * N + f] = static_cast<bf16>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+      }
+    } else {
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int n = n0 + b * 32 + li;
+        if (n < N) ((float*)Cv)[(size_t)row * N + n] = acc[b][r];
+      }
+    }
+  }
+}
+
+// out[t, :] (+)= sum over k, in order, of wts[t, k] * y[row_of_pair[t * top + k], :]
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ row_of_pair,
+                                                          const float* __restrict__ wts, float* __restrict__ out, int top, int D,
+                                                          int accumulate) {
+  const int t = blockIdx.x;
+  for (int d = threadIdx.x; d < D; d += 256) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const int row = row_of_pair[(size_t)t * top + k];
+      if (row >= 0) acc += wts[(size_t)t * top + k] * y[(size_t)row * D + d];
+    }
+    out[(size_t)t * D + d] = accumulate ? out[(size_t)t * D + d] + acc : acc;
+  }
+}
+
 }  // namespace
 
 extern "C" int yalm_moe_route(const void* h, const void* w_router, int dtype, int* ids, float* wts, int T, int D, int E,
@@ -176,5 +366,32 @@ extern "C" int yalm_moe_pair_down(const void* mid, const void* w_down, const int
                                                                         top, D, F, E, accumulate);
   else
     return YALM_ERR_DTYPE;
+  return launch_status();
+}
+
+// The grouped path for many tokens (bfloat16; D and F multiples of 8).  max_tiles = yalm_moe_grouped_tiles(T * top, E);
+// pair_of_row int32 [max_tiles * 128], row_of_pair int32 [T * top], tile_expert int32 [max_tiles], mid bfloat16
+// [max_tiles * 128, F], y float32 [max_tiles * 128, D]: scratch of the caller.
+extern "C" int yalm_moe_grouped_tiles(int n_pairs, int E) { return ceil_div(n_pairs, GR_TM) + E; }
+
+extern "C" int yalm_moe_grouped(const void* h, const void* w_gate, const void* w_up, const void* w_down, const int* ids,
+                                const float* wts, float limit, float alpha, int* pair_of_row, int* row_of_pair,
+                                int* tile_expert, void* mid, float* y, float* out, int T, int top, int D, int F, int E,
+                                int accumulate, hipStream_t stream) {
+  if (T <= 0) return YALM_OK;
+  if (D <= 0 || F <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || (D & 7) || (F & 7) ||
+      ((((uintptr_t)h) | ((uintptr_t)w_gate) | ((uintptr_t)w_up) | ((uintptr_t)w_down) | ((uintptr_t)mid)) & 15))
+    return YALM_ERR_ARG;
+  const long n_pairs = (long)T * top;
+  if (n_pairs > (1l << 30)) return YALM_ERR_ARG;
+  const int max_tiles = yalm_moe_grouped_tiles((int)n_pairs, E);
+  if (max_tiles > 65535) return YALM_ERR_ARG;
+  moe_group_kernel<<<1, GROUP_THREADS, 0, stream>>>(ids, (int)n_pairs, E, max_tiles, pair_of_row, row_of_pair, tile_expert);
+  const size_t lds = (size_t)(GR_TM + GR_TN) * GR_ROW * sizeof(bf16);
+  moe_grouped_kernel<true><<<dim3(ceil_div(F, GR_TN / 2), max_tiles), GR_THREADS, lds, stream>>>(
+      (const bf16*)h, (const bf16*)w_gate, (const bf16*)w_up, tile_expert, pair_of_row, top, mid, F, D, limit, alpha);
+  moe_grouped_kernel<false><<<dim3(ceil_div(D, GR_TN), max_tiles), GR_THREADS, lds, stream>>>(
+      (const bf16*)mid, (const bf16*)w_down, nullptr, tile_expert, pair_of_row, top, y, D, F, 0.f, 0.f);
+  moe_combine_kernel<<<T, 256, 0, stream>>>(y, row_of_pair, wts, out, top, D, accumulate);
   return launch_status();
 }

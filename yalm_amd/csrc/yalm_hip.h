@@ -276,6 +276,16 @@ int yalm_moe_pair_gate_up(const void* h, const void* w_gate, const void* w_up, c
 int yalm_moe_pair_down(const void* mid, const void* w_down, const int* ids, const float* wts, float* out, int T, int top,
                        int D, int F, int E, int dtype, int accumulate, hipStream_t stream);
 
+// The same result for many tokens (bfloat16, D and F multiples of 8): the pairs grouped by expert, each expert's rows
+// padded to tiles of 128, one launch a product over all tiles on the matrix cores.  Scratch of the caller, with
+// max_tiles = yalm_moe_grouped_tiles(T * top, E): pair_of_row int32 [max_tiles * 128], row_of_pair int32 [T * top],
+// tile_expert int32 [max_tiles], mid bfloat16 [max_tiles * 128, F], y float32 [max_tiles * 128, D].
+int yalm_moe_grouped_tiles(int n_pairs, int E);
+int yalm_moe_grouped(const void* h, const void* w_gate, const void* w_up, const void* w_down, const int* ids,
+                     const float* wts, float limit, float alpha, int* pair_of_row, int* row_of_pair, int* tile_expert,
+                     void* mid, float* y, float* out, int T, int top, int D, int F, int E, int accumulate,
+                     hipStream_t stream);
+
 // Yardsticks for the measurement (probes.hip): a kernel that only reads `bytes` bytes once with `workgroups`
 // workgroups (out: 1,024 words of scratch), and a loop of matrix-core instructions on registers (shape 32:
 // v_mfma_f32_32x32x16_bf16, 16: v_mfma_f32_16x16x32_bf16; *flops, host memory, receives the launch's operations).

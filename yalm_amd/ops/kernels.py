@@ -847,6 +847,46 @@ def moe_pair_down(mid, w_down, ids, wts, out, accumulate=False):
     return out
 
 
+
+MOE_GROUP_ROWS = 128           # rows of a tile of the grouped products (csrc/moe.hip)
+
+
+def can_moe_grouped(D, F, dtype):
+    """Whether moe_grouped takes these sizes."""
+    return dtype == torch.bfloat16 and D % 8 == 0 and F % 8 == 0 and not FORCE_SIMPLE
+
+
+def moe_grouped_tiles(n_pairs, n_experts):
+    """Tiles of MOE_GROUP_ROWS rows that the grouped products need at most for n_pairs (token, choice) pairs."""
+    return library.lib().yalm_moe_grouped_tiles(int(n_pairs), int(n_experts))
+
+
+def moe_grouped(h, w_gate, w_up, w_down, ids, wts, limit, alpha, scratch, out, accumulate=False):
+    """What moe_pair_gate_up + moe_pair_down compute, for many tokens (bfloat16): the pairs are grouped by expert on
+    the device and every product is one launch over all experts' tiles on the matrix cores.  scratch(name, shape,
+    dtype) hands out the buffers (pair_of_row, row_of_pair, tile_expert, mid, y)."""
+    T, D = h.shape
+    E, F, _ = w_gate.shape
+    top = ids.shape[1]
+    dt = torch.bfloat16
+    tiles = moe_grouped_tiles(T * top, E)
+    rows = tiles * MOE_GROUP_ROWS
+    pair_of_row = scratch("moe.pair_of_row", (rows,), torch.int32)
+    row_of_pair = scratch("moe.row_of_pair", (T * top,), torch.int32)
+    tile_expert = scratch("moe.tile_expert", (tiles,), torch.int32)
+    mid = scratch("moe.hidden", (rows, F), dt)
+    y = scratch("moe.y", (rows, D), torch.float32)
+    library.check(library.lib().yalm_moe_grouped(
+        _need(h, "h", dt, (T, D)), _need(w_gate, "w_gate", dt, (E, F, D)), _need(w_up, "w_up", dt, (E, F, D)),
+        _need(w_down, "w_down", dt, (E, D, F)), _need(ids, "ids", torch.int32, (T, top)),
+        _need(wts, "wts", torch.float32, (T, top)), float(limit), float(alpha),
+        _need(pair_of_row, "pair_of_row", torch.int32, (rows,)), _need(row_of_pair, "row_of_pair", torch.int32, (T * top,)),
+        _need(tile_expert, "tile_expert", torch.int32, (tiles,)), _need(mid, "mid", dt, (rows, F)),
+        _need(y, "y", torch.float32, (rows, D)), _need(out, "out", torch.float32, (T, D)), T, top, D, F, E,
+        1 if accumulate else 0, _stream()), "moe_grouped")
+    return out
+
+
 def argmax(logits, out):
     R, V = logits.shape
     library.check(library.lib().yalm_argmax(_need(logits, "logits", torch.float32), _need(out, "out", torch.int32, (R,)),

@@ -57,11 +57,13 @@ _SIGNATURES = {
     "yalm_moe_route": (_I, [_P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _P]),
     "yalm_moe_pair_gate_up": (_I, [_P, _P, _P, _P, _F, _F, _P, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_moe_pair_down": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_moe_grouped_tiles": (_I, [_I, _I]),
+    "yalm_moe_grouped": (_I, [_P, _P, _P, _P, _P, _P, _F, _F, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_probe_read": (_I, [_P, ctypes.c_long, _P, _I, _P]),
     "yalm_probe_mfma": (_I, [_I, _I, _I, _P, _P, _P]),
 }
 
-ABI_VERSION = 25
+ABI_VERSION = 26
 
 
 class KernelError(RuntimeError):

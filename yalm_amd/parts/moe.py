@@ -8,12 +8,17 @@ a token's chosen experts, in the order of their scores.
 
 The experts' matrices are stacked at load ([E, F, D], [E, F, D], [E, D, F]); routing happens on the device
 (nothing of it reaches the host, so a decode step stays a captured graph), and every (token, choice) pair is
-served from its expert's weights."""
+served from its expert's weights.  A step of whole prompts with GROUPED_MIN_TOKENS tokens or more (bfloat16) groups
+the pairs by expert instead and multiplies every expert's rows as tiles on the matrix cores, all experts in one
+launch a product."""
 import torch
 
 from ..ops import kernels
 from ..weights.loader import ParamSpec, place
 from .base import Part, part
+
+
+GROUPED_MIN_TOKENS = 48
 
 
 @part("feed_forward", "moe")
@@ -67,6 +72,9 @@ class MixtureOfExperts(Part):
         ids = ws.get("moe.ids", (T, self.top), torch.int32)
         wts = ws.get("moe.weights", (T, self.top), torch.float32)
         kernels.moe_route(h, self.w_router, ids, wts, self.renormalize)
+        if ctx.mode == "prefill" and T >= GROUPED_MIN_TOKENS and kernels.can_moe_grouped(self.dim, self.hidden, h.dtype):
+            return kernels.moe_grouped(h, self.w_gate, self.w_up, self.w_down, ids, wts, self.limit, self.alpha, ws.get,
+                                       out, accumulate)
         mid = ws.get("moe.hidden", (T * self.top, self.hidden), h.dtype)
         kernels.moe_pair_gate_up(h, self.w_gate, self.w_up, ids, self.limit, self.alpha, mid)
         kernels.moe_pair_down(mid, self.w_down, ids, wts, out, accumulate)
