@@ -45,6 +45,13 @@ def test_norm_add(R_, D, out_dtype):
     assert torch.allclose(xd.cpu().to(F64), want, rtol=1e-5, atol=1e-5)
     if h is not None:
         assert torch.equal(h.cpu(), xd.cpu().to(out_dtype))
+    if h is not None:                                           # the norm that reads the stream next, done on the way
+        w2 = 1.0 + 0.1 * randn(D, seed=13)
+        xd = x.to(DEV)
+        kernels.norm_add(y.to(DEV), w.to(DEV), 1e-5, xd, h, next_norm=(w2.to(DEV), 3e-6))
+        assert torch.allclose(xd.cpu().to(F64), want, rtol=1e-5, atol=1e-5)
+        tol = 1e-5 if out_dtype == torch.float32 else 1e-2
+        assert torch.allclose(h.cpu().to(F64), P.rms_norm(want, w2.to(F64), 3e-6), rtol=tol, atol=tol)
     wb = w.to(torch.bfloat16)                                   # bfloat16 norm weights
     xd = x.to(DEV)
     kernels.norm_add(y.to(DEV), wb.to(DEV), 1e-5, xd)
@@ -133,6 +140,10 @@ def test_router_and_experts(dtype, T, D, E, top):
     kernels.moe_route(h.to(DEV), w["router"].to(DEV), ids, wts)
     assert torch.equal(ids.cpu().long(), chosen)
     assert torch.allclose(wts.cpu().to(F64), weight, rtol=1e-5, atol=1e-7)
+    logits = (h.to(F64) @ w["router"].to(F64).T).float().to(DEV)          # the same choice from ready logits
+    ids2, wts2 = torch.zeros_like(ids), torch.zeros_like(wts)
+    kernels.moe_select(logits, ids2, wts2)
+    assert torch.equal(ids2, ids) and torch.allclose(wts2, wts, rtol=1e-5, atol=1e-7)
     kernels.moe_route(h.to(DEV), w["router"].to(DEV), ids, wts, renormalize=True)
     assert torch.allclose(wts.cpu().to(F64), weight / weight.sum(-1, keepdim=True), rtol=1e-5, atol=1e-7)
     kernels.moe_route(h.to(DEV), w["router"].to(DEV), ids, wts)

@@ -8,7 +8,7 @@
 //    head-shaped rows that the rotation kernel reads (query rotated parts scaled, key, value).
 //  * yalm_head_matmul: out[t, h, :] = scale * in[t, h, :] Wt[h] for every head, Wt [H, K, N]
 //    (optionally times sigmoid(gate)): the two per-head products (W_uk^T on queries, W_uv on results).
-//    float32 arithmetic; a workgroup owns a head and 16 tokens, a lane a column of the result.
+//    float32 arithmetic; a workgroup owns 16 tokens and 64 columns of a head's result, a lane a column.
 #include "common.h"
 #include "yalm_hip.h"
 
@@ -36,9 +36,20 @@ __global__ __launch_bounds__(HM_THREADS) void head_matmul_kernel(const TI* __res
   const int tg = threadIdx.x / WAVE;        // a wave takes 4 of the 16 tokens
   const int lane = threadIdx.x % WAVE;
   const TW* w = wt + (size_t)h * K * N;
-  for (int n = lane; n < N; n += WAVE) {
+  const int n = blockIdx.z * WAVE + lane;          // a workgroup owns 64 columns of the head's result
+  if (n < N) {
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int k = 0; k < K; ++k) {
+    int k = 0;
+    for (; k + 8 <= K; k += 8) {                     // eight loads in flight, then their products
+      float wv[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) wv[i] = to_f32(w[(size_t)(k + i) * N + n]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] += tile[tg * 4 + j][k + i] * wv[i];
+    }
+    for (; k < K; ++k) {
       const float wv = to_f32(w[(size_t)k * N + n]);
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[j] += tile[tg * 4 + j][k] * wv;
@@ -100,7 +111,7 @@ template <typename TI, typename TW, typename TO>
 int head_matmul_launch(const void* in, long in_row, int in_head, int in_off, const void* wt, void* out, long out_row,
                        int out_head, int out_off, float scale, const float* gate, long gate_row, int T, int H, int K,
                        int N, hipStream_t stream) {
-  dim3 grid(ceil_div(T, HM_TOK), H);
+  dim3 grid(ceil_div(T, HM_TOK), H, ceil_div(N, WAVE));
   head_matmul_kernel<TI, TW, TO><<<grid, HM_THREADS, 0, stream>>>((const TI*)in, in_row, in_head, in_off, (const TW*)wt,
                                                                   (TO*)out, out_row, out_head, out_off, scale, gate,
                                                                   gate_row, T, K, N);

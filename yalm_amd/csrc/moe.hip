@@ -43,15 +43,20 @@ __device__ __forceinline__ float dot_row<bf16>(const bf16* __restrict__ w, const
   return acc;
 }
 
+// logits given (w null, h = float32 logits [T, E]) or made here, a dot product a wave at a time
 template <typename T>
 __global__ __launch_bounds__(WAVE) void moe_route_kernel(const T* __restrict__ h, const T* __restrict__ w, int* __restrict__ ids,
                                                          float* __restrict__ wts, int D, int E, int top, int renorm) {
   __shared__ float score[MOE_MAX_EXPERTS];
   const int t = blockIdx.x, lane = threadIdx.x;
-  const T* x = h + (size_t)t * D;
-  for (int e = 0; e < E; ++e) {
-    const float z = wave_sum(dot_row<T>(w + (size_t)e * D, x, D, lane));
-    if (lane == 0) score[e] = z;
+  if (w == nullptr) {
+    for (int e = lane; e < E; e += WAVE) score[e] = to_f32(h[(size_t)t * E + e]);
+  } else {
+    const T* x = h + (size_t)t * D;
+    for (int e = 0; e < E; ++e) {
+      const float z = wave_sum(dot_row<T>(w + (size_t)e * D, x, D, lane));
+      if (lane == 0) score[e] = z;
+    }
   }
   __syncthreads();
   float m = -3.0e38f;
@@ -332,6 +337,14 @@ extern "C" int yalm_moe_route(const void* h, const void* w_router, int dtype, in
     moe_route_kernel<float><<<T, WAVE, 0, stream>>>((const float*)h, (const float*)w_router, ids, wts, D, E, top, renorm);
   else
     return YALM_ERR_DTYPE;
+  return launch_status();
+}
+
+extern "C" int yalm_moe_select(const float* logits, int* ids, float* wts, int T, int E, int top, int renorm,
+                               hipStream_t stream) {
+  if (T <= 0) return YALM_OK;
+  if (E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > E) return YALM_ERR_ARG;
+  moe_route_kernel<float><<<T, WAVE, 0, stream>>>(logits, nullptr, ids, wts, E, E, top, renorm);
   return launch_status();
 }
 

@@ -16,30 +16,39 @@ __global__ __launch_bounds__(ROW_THREADS) void cast_kernel(const float* __restri
   for (; i < n; i += step) out[i] = from_f32<T>(x[i]);
 }
 
-// x[r] += y[r] * rsqrt(mean(y[r]^2) + eps) * w; h[r] = T(x[r]) if h is given
-template <typename W, typename T>
-__global__ __launch_bounds__(ROW_THREADS) void norm_add_kernel(const float* __restrict__ y, const W* __restrict__ w, float eps,
-                                                               float* __restrict__ x, T* __restrict__ h, int D) {
-  __shared__ float red[ROW_WAVES];
+// x[r] += y[r] * rsqrt(mean(y[r]^2) + eps) * w; if h is given: h[r] = T(x[r]), or with next_w the norm that reads
+// the stream next, h[r] = T(x[r] * rsqrt(mean(x[r]^2) + next_eps) * next_w)
+template <typename W, typename T, int NT>
+__global__ __launch_bounds__(NT) void norm_add_kernel(const float* __restrict__ y, const W* __restrict__ w, float eps,
+                                                      float* __restrict__ x, T* __restrict__ h, const float* __restrict__ next_w,
+                                                      float next_eps, int D) {
+  __shared__ float red[NT / WAVE];
   const size_t row = (size_t)blockIdx.x * D;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < D; i += ROW_THREADS) {
+  for (int i = threadIdx.x; i < D; i += NT) {
     const float v = y[row + i];
     ss += v * v;
   }
-  ss = block_sum<ROW_WAVES>(ss, red);
+  ss = block_sum<NT / WAVE>(ss, red);
   const float scale = 1.0f / sqrtf(ss / (float)D + eps);
-  for (int i = threadIdx.x; i < D; i += ROW_THREADS) {
+  float ss2 = 0.f;
+  for (int i = threadIdx.x; i < D; i += NT) {
     const float v = x[row + i] + y[row + i] * scale * to_f32(w[i]);
     x[row + i] = v;
-    if (h != nullptr) h[row + i] = from_f32<T>(v);
+    ss2 += v * v;
+    if (h != nullptr && next_w == nullptr) h[row + i] = from_f32<T>(v);
   }
+  if (h == nullptr || next_w == nullptr) return;
+  ss2 = block_sum<NT / WAVE>(ss2, red);
+  const float scale2 = 1.0f / sqrtf(ss2 / (float)D + next_eps);
+  for (int i = threadIdx.x; i < D; i += NT) h[row + i] = from_f32<T>(x[row + i] * scale2 * next_w[i]);   // its own stores
 }
 
 // out = a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps) over the row
-template <typename T>
-__global__ __launch_bounds__(ROW_THREADS) void polynorm_kernel(const float* __restrict__ z, const float* __restrict__ coef, float eps,
-                                                               T* __restrict__ out, int F) {
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void polynorm_kernel(const float* __restrict__ z, const float* __restrict__ coef, float eps,
+                                                      T* __restrict__ out, int F) {
+  constexpr int ROW_THREADS = NT, ROW_WAVES = NT / WAVE;
   __shared__ float red[ROW_WAVES];
   const size_t row = (size_t)blockIdx.x * F;
   float s2 = 0.f, s4 = 0.f, s6 = 0.f;
@@ -77,32 +86,43 @@ extern "C" int yalm_cast(const float* x, void* out, long n, int out_dtype, hipSt
   return launch_status();
 }
 
+template <typename W, typename T>
+static int norm_add_launch(const float* y, const void* w, float eps, float* x, void* h, const float* next_w, float next_eps,
+                           int R, int D, hipStream_t stream) {
+  if (D >= 2048)
+    norm_add_kernel<W, T, 1024><<<R, 1024, 0, stream>>>(y, (const W*)w, eps, x, (T*)h, next_w, next_eps, D);
+  else
+    norm_add_kernel<W, T, 256><<<R, 256, 0, stream>>>(y, (const W*)w, eps, x, (T*)h, next_w, next_eps, D);
+  return launch_status();
+}
+
 extern "C" int yalm_norm_add(const float* y, const void* w, int w_dtype, float eps, float* x, void* h_out, int h_dtype,
-                             int R, int D, hipStream_t stream) {
+                             const float* next_w, float next_eps, int R, int D, hipStream_t stream) {
   if (R <= 0) return YALM_OK;
   if (D <= 0) return YALM_ERR_ARG;
   if (w_dtype != YALM_F32 && w_dtype != YALM_BF16) return YALM_ERR_DTYPE;
   if (h_out != nullptr && h_dtype != YALM_F32 && h_dtype != YALM_BF16) return YALM_ERR_DTYPE;
   const bool hb = h_out != nullptr && h_dtype == YALM_BF16;
-  if (w_dtype == YALM_F32) {
-    if (hb) norm_add_kernel<float, bf16><<<R, ROW_THREADS, 0, stream>>>(y, (const float*)w, eps, x, (bf16*)h_out, D);
-    else norm_add_kernel<float, float><<<R, ROW_THREADS, 0, stream>>>(y, (const float*)w, eps, x, (float*)h_out, D);
-  } else {
-    if (hb) norm_add_kernel<bf16, bf16><<<R, ROW_THREADS, 0, stream>>>(y, (const bf16*)w, eps, x, (bf16*)h_out, D);
-    else norm_add_kernel<bf16, float><<<R, ROW_THREADS, 0, stream>>>(y, (const bf16*)w, eps, x, (float*)h_out, D);
-  }
-  return launch_status();
+  if (w_dtype == YALM_F32)
+    return hb ? norm_add_launch<float, bf16>(y, w, eps, x, h_out, next_w, next_eps, R, D, stream)
+              : norm_add_launch<float, float>(y, w, eps, x, h_out, next_w, next_eps, R, D, stream);
+  return hb ? norm_add_launch<bf16, bf16>(y, w, eps, x, h_out, next_w, next_eps, R, D, stream)
+            : norm_add_launch<bf16, float>(y, w, eps, x, h_out, next_w, next_eps, R, D, stream);
 }
 
 extern "C" int yalm_polynorm(const float* z, const float* coef, float eps, void* out, int out_dtype, int R, int F,
                              hipStream_t stream) {
   if (R <= 0) return YALM_OK;
   if (F <= 0) return YALM_ERR_ARG;
-  if (out_dtype == YALM_BF16)
-    polynorm_kernel<bf16><<<R, ROW_THREADS, 0, stream>>>(z, coef, eps, (bf16*)out, F);
-  else if (out_dtype == YALM_F32)
-    polynorm_kernel<float><<<R, ROW_THREADS, 0, stream>>>(z, coef, eps, (float*)out, F);
-  else
+  const bool wide = F >= 2048;
+  if (out_dtype == YALM_BF16) {
+    if (wide) polynorm_kernel<bf16, 1024><<<R, 1024, 0, stream>>>(z, coef, eps, (bf16*)out, F);
+    else polynorm_kernel<bf16, 256><<<R, 256, 0, stream>>>(z, coef, eps, (bf16*)out, F);
+  } else if (out_dtype == YALM_F32) {
+    if (wide) polynorm_kernel<float, 1024><<<R, 1024, 0, stream>>>(z, coef, eps, (float*)out, F);
+    else polynorm_kernel<float, 256><<<R, 256, 0, stream>>>(z, coef, eps, (float*)out, F);
+  } else {
     return YALM_ERR_DTYPE;
+  }
   return launch_status();
 }

@@ -239,12 +239,13 @@ int yalm_token_prob(const float* logits, const int* index, float* prob, int R, i
 
 // Layers that norm a sublayer's OUTPUT before it joins the residual stream (postnorm.hip).
 // yalm_cast: out[i] = dtype(x[i]).  yalm_norm_add: x[r, :] += y[r, :] * rsqrt(mean(y[r]^2) + eps) * w, and if h_out is
-// given h_out[r, :] = dtype(x_new[r, :]) (the next sublayer's input).  yalm_polynorm: out[r, :] = a N(z) + b N(z^2) +
+// given h_out[r, :] = dtype(x_new[r, :]) (the next sublayer's input), or, with next_w (float32 [D]: the weights of the
+// norm that reads the stream next), dtype(x_new[r, :] * rsqrt(mean(x_new[r]^2) + next_eps) * next_w).  yalm_polynorm: out[r, :] = a N(z) + b N(z^2) +
 // c N(z^3) + e with powers element by element, N(v) = v / sqrt(mean(v^2) + eps) over the row and coef = {a, b, c, e}
 // (float32, on the device).
 int yalm_cast(const float* x, void* out, long n, int out_dtype, hipStream_t stream);
-int yalm_norm_add(const float* y, const void* w, int w_dtype, float eps, float* x, void* h_out, int h_dtype, int R, int D,
-                  hipStream_t stream);
+int yalm_norm_add(const float* y, const void* w, int w_dtype, float eps, float* x, void* h_out, int h_dtype,
+                  const float* next_w, float next_eps, int R, int D, hipStream_t stream);
 int yalm_polynorm(const float* z, const float* coef, float eps, void* out, int out_dtype, int R, int F,
                   hipStream_t stream);
 
@@ -271,6 +272,8 @@ int yalm_latent_pack(const float* proj, long proj_row, int q_head, int q_rot_off
 // -limit, limit) (limit <= 0: unclamped); out float32 [T, D] = (accumulate: out +) sum_k wts[t, k] * w_down[ids[t, k]] mid[t, k], k in order.
 int yalm_moe_route(const void* h, const void* w_router, int dtype, int* ids, float* wts, int T, int D, int E, int top,
                    int renorm, hipStream_t stream);
+// The same choice from logits that a product has made already (float32 [T, E]).
+int yalm_moe_select(const float* logits, int* ids, float* wts, int T, int E, int top, int renorm, hipStream_t stream);
 int yalm_moe_pair_gate_up(const void* h, const void* w_gate, const void* w_up, const int* ids, float limit, float alpha,
                           void* mid, int T, int top, int D, int F, int E, int dtype, hipStream_t stream);
 int yalm_moe_pair_down(const void* mid, const void* w_down, const int* ids, const float* wts, float* out, int T, int top,

@@ -731,16 +731,22 @@ def cast(x, out):
     return out
 
 
-def norm_add(y, weight, eps, x, h_out=None):
+def norm_add(y, weight, eps, x, h_out=None, next_norm=None):
     """x += y * rsqrt(mean(y^2) + eps) * weight, row by row (x, y float32 [R, D]); h_out (optional, [R, D] in the
-    compute dtype) receives the new x: the input of the sublayer that follows."""
+    compute dtype) receives the new x: the input of the sublayer that follows; with next_norm = (float32 weights [D],
+    eps) it receives the RMS norm of the new x with those weights instead (the norm that reads the stream next)."""
     R, D = y.shape
     p_h, h_code = None, 0
     if h_out is not None:
         p_h, h_code = _need(h_out, "h_out", None, (R, D)), dtype_code(h_out.dtype)
+    p_n, n_eps = None, 0.0
+    if next_norm is not None:
+        if h_out is None:
+            raise ValueError("norm_add: the next norm's output needs h_out")
+        p_n, n_eps = _need(next_norm[0], "next norm weight", torch.float32, (D,)), float(next_norm[1])
     library.check(library.lib().yalm_norm_add(
         _need(y, "y", torch.float32, (R, D)), _need(weight, "weight", None, (D,)), dtype_code(weight.dtype), float(eps),
-        _need(x, "x", torch.float32, (R, D)), p_h, h_code, R, D, _stream()), "norm_add")
+        _need(x, "x", torch.float32, (R, D)), p_h, h_code, p_n, n_eps, R, D, _stream()), "norm_add")
     return x
 
 
@@ -819,6 +825,17 @@ def moe_route(h, w_router, ids, wts, renormalize=False):
         _need(h, "h", None, (T, D)), _need(w_router, "w_router", h.dtype, (E, D)), dtype_code(h.dtype),
         _need(ids, "ids", torch.int32, (T, top)), _need(wts, "wts", torch.float32, (T, top)), T, D, E, top,
         1 if renormalize else 0, _stream()), "moe_route")
+
+
+def moe_select(logits, ids, wts, renormalize=False):
+    """moe_route from logits that a product has made already (float32 [T, E])."""
+    T, E = logits.shape
+    top = ids.shape[1]
+    if not 0 < top <= E or E > MOE_MAX_EXPERTS:
+        raise ValueError("moe_select: %d of %d experts is not offered (at most %d experts)" % (top, E, MOE_MAX_EXPERTS))
+    library.check(library.lib().yalm_moe_select(
+        _need(logits, "logits", torch.float32, (T, E)), _need(ids, "ids", torch.int32, (T, top)),
+        _need(wts, "wts", torch.float32, (T, top)), T, E, top, 1 if renormalize else 0, _stream()), "moe_select")
 
 
 def moe_pair_gate_up(h, w_gate, w_up, ids, limit, alpha, mid):

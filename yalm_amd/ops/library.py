@@ -49,12 +49,13 @@ _SIGNATURES = {
     "yalm_gemm_scaled": (_I, [_P, _P, _P, _P, ctypes.c_long, _I, _I, _I, _I, _I, _P, _I, _F, _P]),
     "yalm_gemm_partial_scaled": (_I, [_P, _P, _P, ctypes.c_long, _I, _I, _I, _P, _P, _I, _F, _P]),
     "yalm_cast": (_I, [_P, _P, ctypes.c_long, _I, _P]),
-    "yalm_norm_add": (_I, [_P, _P, _I, _F, _P, _P, _I, _I, _I, _P]),
+    "yalm_norm_add": (_I, [_P, _P, _I, _F, _P, _P, _I, _P, _F, _I, _I, _P]),
     "yalm_polynorm": (_I, [_P, _P, _F, _P, _I, _I, _I, _P]),
     "yalm_head_matmul": (_I, [_P, _I, ctypes.c_long, _I, _I, _P, _I, _P, _I, ctypes.c_long, _I, _I, _F, _P, ctypes.c_long,
                               _I, _I, _I, _I, _P]),
     "yalm_latent_pack": (_I, [_P, ctypes.c_long, _I, _I, _I, _P, _I, _F, _F, _P, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_moe_route": (_I, [_P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "yalm_moe_select": (_I, [_P, _P, _P, _I, _I, _I, _I, _P]),
     "yalm_moe_pair_gate_up": (_I, [_P, _P, _P, _P, _F, _F, _P, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_moe_pair_down": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_moe_grouped_tiles": (_I, [_I, _I]),
@@ -63,7 +64,7 @@ _SIGNATURES = {
     "yalm_probe_mfma": (_I, [_I, _I, _I, _P, _P, _P]),
 }
 
-ABI_VERSION = 26
+ABI_VERSION = 27
 
 
 class KernelError(RuntimeError):

@@ -85,14 +85,18 @@ class PostNormResidualBlock(Part):
         else:
             h = kernels.cast(x, ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype))
         hand_on = None if same or not isinstance(next_norm, StreamInput) else ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype)
+        # the last layer of a decode step leaves the final norm's output for the head
+        final = next_norm if ctx.mode == "decode" and hasattr(next_norm, "fused") else None
+        if final is not None:
+            hand_on = ctx.ws.get("block.normed", (T, self.dim), ctx.act_dtype)
         y = ctx.ws.get("block.y", (T, self.dim), torch.float32)
         self.mixer.forward_to(h, y, ctx, line, writes_cache)
         if self.feed_forward is None:
-            self.mixer_norm.add_normed(y, x, ctx, h_out=hand_on)
+            self.mixer_norm.add_normed(y, x, ctx, h_out=hand_on, next_norm=final)
         else:
             h = x if same else ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype)
             self.mixer_norm.add_normed(y, x, ctx, h_out=None if same else h)
             self.feed_forward.forward_to(h, y, ctx)
-            self.feed_forward_norm.add_normed(y, x, ctx, h_out=hand_on)
+            self.feed_forward_norm.add_normed(y, x, ctx, h_out=hand_on, next_norm=final)
         if hand_on is not None:
             ctx.normed[id(next_norm)] = (hand_on, None, None)

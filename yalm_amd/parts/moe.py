@@ -71,7 +71,9 @@ class MixtureOfExperts(Part):
         ws = ctx.ws
         ids = ws.get("moe.ids", (T, self.top), torch.int32)
         wts = ws.get("moe.weights", (T, self.top), torch.float32)
-        kernels.moe_route(h, self.w_router, ids, wts, self.renormalize)
+        logits = ws.get("moe.logits", (T, self.n_experts), torch.float32)        # products exact, sums in float32
+        self._gemm(ctx, h, self.w_router, logits, kernels.EPI_STORE_F32)
+        kernels.moe_select(logits, ids, wts, self.renormalize)
         if ctx.mode == "prefill" and T >= GROUPED_MIN_TOKENS and kernels.can_moe_grouped(self.dim, self.hidden, h.dtype):
             return kernels.moe_grouped(h, self.w_gate, self.w_up, self.w_down, ids, wts, self.limit, self.alpha, ws.get,
                                        out, accumulate)

@@ -34,6 +34,7 @@ class RMSNorm(Part):
     def forward(self, x, out, ctx, row_index=None):
         return kernels.rmsnorm(x, self.weight, out, self.eps, row_index)
 
-    def add_normed(self, y, x, ctx, h_out=None):
-        """x += norm(y) (both float32 [T, dim]); h_out, if given, receives the new x in the compute dtype."""
-        return kernels.norm_add(y, self.weight, self.eps, x, h_out)
+    def add_normed(self, y, x, ctx, h_out=None, next_norm=None):
+        """x += norm(y) (both float32 [T, dim]); h_out, if given, receives the new x in the compute dtype, or with
+        next_norm (a norm that offers fused()) that norm's output for the new x."""
+        return kernels.norm_add(y, self.weight, self.eps, x, h_out, None if next_norm is None else next_norm.fused())
