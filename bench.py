@@ -331,6 +331,9 @@ def bench_design(args):
             ctx_len = engine.length(slots[0]) - args.steps / 2.0
             kv = sum(g.bytes_per_token() * (min(ctx_len, g.window) if g.window else ctx_len) for g in engine.cache.kv_groups) * B
             step_bytes = model.weight_bytes() + kv
+            for part in model.all_parts():              # a batch reads up to batch x top experts, not one token's top
+                if hasattr(part, "n_experts"):
+                    step_bytes += (min(part.n_experts, B * part.top) - part.top) * 3 * part.hidden * part.dim * part.w_down.element_size()
             r = {"prefill_tokens": T, "prefill_ms": round(prefill_s * 1e3, 3), "prefill_tok_s": round(T / prefill_s, 1),
                  "decode_batch": B, "decode_context": int(ctx_len), "decode_ms_per_step": round(step_s * 1e3, 4),
                  "decode_tok_s": round(B / step_s, 1), "decode_step_MB": round(step_bytes / 1e6, 1),

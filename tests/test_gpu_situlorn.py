@@ -100,6 +100,32 @@ def test_head_matmul(types, T, H, K, N):
         assert (block[:, :, :out_off] == 7.0).all() and (block[:, :, out_off + N:] == 7.0).all()     # nothing else is touched
 
 
+@pytest.mark.parametrize("types", ["ff", "bb", "fb"])
+@pytest.mark.parametrize("T,H,K,N", [(64, 1, 8, 3), (130, 3, 32, 40), (300, 2, 96, 130), (257, 5, 200, 64)])
+def test_head_matmul_on_the_matrix_cores(types, T, H, K, N):
+    """The product of a step of many tokens: the same numbers as float64 on the inputs rounded to bfloat16."""
+    from yalm_amd.ops import kernels
+    dt = {"f": torch.float32, "b": torch.bfloat16}
+    ti, to = dt[types[0]], dt[types[1]]
+    src_head, src_off, out_head, out_off = K + 16, 8, N + 10, 3
+    src = randn(T, H * src_head + 8, seed=15).to(ti)
+    wt = randn(H, K, N, seed=16, scale=K ** -0.5).to(torch.bfloat16)
+    gate = randn(T, H * N + 5, seed=17)
+    for use_gate in (False, True):
+        out = torch.full((T, H * out_head + 1), 7.0, dtype=to, device=DEV)
+        g = gate.to(DEV)[:, 3:] if use_gate else None
+        kernels.head_matmul(src.to(DEV), src_head, src_off, wt.to(DEV), out, out_head, out_off, scale=0.37, gate=g,
+                            wt_nk=wt.transpose(1, 2).contiguous().to(DEV))
+        s64 = src.to(torch.bfloat16).to(F64)[:, :H * src_head].reshape(T, H, src_head)[:, :, src_off:src_off + K]
+        want = 0.37 * torch.einsum("thk,hkn->thn", s64, wt.to(F64))
+        if use_gate:
+            want = want * torch.sigmoid(gate.to(F64)[:, 3:3 + H * N].reshape(T, H, N))
+        tol = 1e-4 if to == torch.float32 else 2e-2
+        block = out.cpu().to(F64)[:, :H * out_head].reshape(T, H, out_head)
+        assert torch.allclose(block[:, :, out_off:out_off + N], want, rtol=tol, atol=tol)
+        assert (block[:, :, :out_off] == 7.0).all() and (block[:, :, out_off + N:] == 7.0).all()
+
+
 @pytest.mark.parametrize("T,H,d,r,rank", [(1, 1, 4, 2, 6), (9, 3, 16, 8, 40), (70, 2, 8, 0, 16)])
 def test_latent_pack(T, H, d, r, rank):
     from yalm_amd.ops import kernels

@@ -145,7 +145,7 @@ __global__ __launch_bounds__(PAIR_WAVES * WAVE) void moe_pair_down_kernel(const 
 // tile_expert[tile] (-1: behind the last used tile).  The order of an expert's rows among themselves is not
 // fixed, and no result depends on it: a row of a product depends on that row alone.
 // ---------------------------------------------------------------------------
-constexpr int GR_TM = 128, GR_TN = 128, GR_TK = 64, GR_ROW = GR_TK + 8, GR_THREADS = 256;
+constexpr int GR_TM = 128, GR_TN = 256, GR_TK = 64, GR_ROW = GR_TK + 8, GR_THREADS = 256;
 constexpr int GROUP_THREADS = 1024;
 
 __global__ __launch_bounds__(GROUP_THREADS) void moe_group_kernel(const int* __restrict__ ids, int n_pairs, int E, int max_tiles,
@@ -190,12 +190,13 @@ __global__ __launch_bounds__(GROUP_THREADS) void moe_group_kernel(const int* __r
 typedef __attribute__((ext_vector_type(8))) __bf16 gr_bf16x8;
 typedef __attribute__((ext_vector_type(16))) float gr_f32x16;
 
-// A tile of GR_TM rows x GR_TN weight rows, 4 waves, each 32 rows x all weight rows (v_mfma_f32_32x32x16_bf16:
-// operand rows = lane % 32, 8 k a lane at k offset 8 * (lane / 32); C: column = lane % 32, rows 8 (r / 4) + 4
-// (lane / 32) + r % 4).  One LDS buffer, the next k tile waits in registers.
-// GATED: A rows are gathered (row -> pair -> token), the weight rows are 64 gate rows and the 64 up rows of the
-// same hidden columns, and the epilogue writes mid[row, f] = act(g, u).  Else: A = mid rows as they lie, the
-// weight rows are 128 rows of the expert's down matrix, and the epilogue stores float32 out[row, n].
+// A tile of GR_TM rows x GR_TN weight rows, 4 waves in 2 x 2, each 64 rows x 128 weight rows: six fragment reads
+// for eight matrix instructions (v_mfma_f32_32x32x16_bf16: operand rows = lane % 32, 8 k a lane at k offset
+// 8 * (lane / 32); C: column = lane % 32, rows 8 (r / 4) + 4 (lane / 32) + r % 4).  One LDS buffer, the next k tile
+// waits in registers.
+// GATED: A rows are gathered (row -> pair -> token); a wave's 128 weight rows are 64 gate rows and the 64 up rows of
+// the same hidden columns, and the epilogue writes mid[row, f] = act(g, u).  Else: A = mid rows as they lie, the
+// weight rows are 256 rows of the expert's down matrix, and the epilogue stores float32 out[row, n].
 template <bool GATED>
 __global__ __launch_bounds__(GR_THREADS, 2) void moe_grouped_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W0,
                                                                     const bf16* __restrict__ W1, const int* __restrict__ tile_expert,
@@ -207,11 +208,12 @@ __global__ __launch_bounds__(GR_THREADS, 2) void moe_grouped_kernel(const bf16* 
   bf16* As = reinterpret_cast<bf16*>(smem_raw);       // [GR_TM][GR_ROW]
   bf16* Ws = As + GR_TM * GR_ROW;                      // [GR_TN][GR_ROW]
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int wm = wave / 2, wn = wave % 2;
   const int li = lane % 32, lh = lane / 32;
   const int m0 = blockIdx.y * GR_TM;
   const int n0 = blockIdx.x * (GATED ? GR_TN / 2 : GR_TN);      // first output column of the tile
   constexpr int RPP = GR_THREADS / 8;                  // 32 rows a pass
-  constexpr int LA = GR_TM / RPP, LB = GR_TN / RPP;    // 4 chunks of 16 bytes a thread and operand
+  constexpr int LA = GR_TM / RPP, LB = GR_TN / RPP;    // chunks of 16 bytes a thread and operand
   const int lrow = tid / 8, lk = (tid % 8) * 8;
   const bf16* ap[LA];
   const bf16* wp[LB];
@@ -219,23 +221,18 @@ __global__ __launch_bounds__(GR_THREADS, 2) void moe_grouped_kernel(const bf16* 
 #pragma unroll
   for (int p = 0; p < LA; ++p) {
     const int row = m0 + lrow + RPP * p;
-    if (GATED) {
-      const int pair = pair_of_row[row];
-      aok[p] = pair >= 0;
-      ap[p] = A + (size_t)(aok[p] ? pair / top : 0) * K + lk;
-    } else {
-      aok[p] = pair_of_row[row] >= 0;
-      ap[p] = A + (size_t)row * K + lk;
-    }
+    const int pair = pair_of_row[row];
+    aok[p] = pair >= 0;
+    ap[p] = A + (size_t)(GATED ? (aok[p] ? pair / top : 0) : row) * K + lk;
   }
 #pragma unroll
   for (int p = 0; p < LB; ++p) {
     const int j = lrow + RPP * p;                      // row of the weight tile
     int n;
     const bf16* base;
-    if (GATED) {
-      n = n0 + (j % (GR_TN / 2));
-      base = j < GR_TN / 2 ? W0 : W1;
+    if (GATED) {                                       // [gate 0..63 | up 0..63 | gate 64..127 | up 64..127]
+      n = n0 + (j / 128) * 64 + j % 64;
+      base = (j / 64) % 2 ? W1 : W0;
     } else {
       n = n0 + j;
       base = W0;
@@ -243,11 +240,13 @@ __global__ __launch_bounds__(GR_THREADS, 2) void moe_grouped_kernel(const bf16* 
     wok[p] = n < N;
     wp[p] = base + ((size_t)e * N + (wok[p] ? n : 0)) * K + lk;
   }
-  gr_f32x16 acc[4];
+  gr_f32x16 acc[2][4];
 #pragma unroll
-  for (int b = 0; b < 4; ++b)
+  for (int a = 0; a < 2; ++a)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[b][r] = 0.f;
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
   const gr_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   gr_bf16x8 ra[LA], rw[LB];
   const int nk = (K + GR_TK - 1) / GR_TK;
@@ -275,36 +274,44 @@ __global__ __launch_bounds__(GR_THREADS, 2) void moe_grouped_kernel(const bf16* 
     }
 #pragma unroll
     for (int ks = 0; ks < GR_TK / 16; ++ks) {
-      const gr_bf16x8 fa = *reinterpret_cast<const gr_bf16x8*>(&As[(wave * 32 + li) * GR_ROW + ks * 16 + lh * 8]);
+      gr_bf16x8 fa[2], fw[4];
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const gr_bf16x8 fw = *reinterpret_cast<const gr_bf16x8*>(&Ws[(b * 32 + li) * GR_ROW + ks * 16 + lh * 8]);
-        acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fw, acc[b], 0, 0, 0);
-      }
+      for (int a = 0; a < 2; ++a)
+        fa[a] = *reinterpret_cast<const gr_bf16x8*>(&As[(wm * 64 + a * 32 + li) * GR_ROW + ks * 16 + lh * 8]);
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+        fw[b] = *reinterpret_cast<const gr_bf16x8*>(&Ws[(wn * 128 + b * 32 + li) * GR_ROW + ks * 16 + lh * 8]);
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[a], fw[b], acc[a][b], 0, 0, 0);
     }
     __syncthreads();
   }
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int row = m0 + wave * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
-    if (pair_of_row[row] < 0) continue;
-    if (GATED) {
+  for (int a = 0; a < 2; ++a) {
 #pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const int f = n0 + b * 32 + li;
-        if (f >= N) continue;
-        float g = acc[b][r], u = acc[b + 2][r];
-        if (limit > 0.f) {
-          g = fminf(g, limit);
-          u = fminf(fmaxf(u, -limit), limit);
+    for (int r = 0; r < 16; ++r) {
+      const int row = m0 + wm * 64 + a * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+      if (pair_of_row[row] < 0) continue;
+      if (GATED) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          const int f = n0 + wn * 64 + b * 32 + li;
+          if (f >= N) continue;
+          float g = acc[a][b][r], u = acc[a][b + 2][r];
+          if (limit > 0.f) {
+            g = fminf(g, limit);
+            u = fminf(fmaxf(u, -limit), limit);
+          }
+          ((bf16*)Cv)[(size_t)row * N + f] = static_cast<bf16>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
         }
-        ((bf16*)Cv)[(size_t)row * N + f] = static_cast<bf16>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
-      }
-    } else {
+      } else {
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const int n = n0 + b * 32 + li;
-        if (n < N) ((float*)Cv)[(size_t)row * N + n] = acc[b][r];
+        for (int b = 0; b < 4; ++b) {
+          const int n = n0 + wn * 128 + b * 32 + li;
+          if (n < N) ((float*)Cv)[(size_t)row * N + n] = acc[a][b][r];
+        }
       }
     }
   }

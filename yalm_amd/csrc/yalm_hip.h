@@ -261,6 +261,12 @@ int yalm_polynorm(const float* z, const float* coef, float eps, void* out, int o
 int yalm_head_matmul(const void* in, int in_dtype, long in_row, int in_head, int in_off, const void* wt, int w_dtype,
                      void* out, int out_dtype, long out_row, int out_head, int out_off, float scale, const float* gate,
                      long gate_row, int T, int H, int K, int N, hipStream_t stream);
+// yalm_head_matmul for many tokens on the matrix cores: wn is wt with its last two axes exchanged, bfloat16 [H, N, K]; the
+// input (float32 or bfloat16) is rounded to bfloat16, the sums are float32, out float32 or bfloat16.  K must be a multiple
+// of 8 and in_row, in_head, in_off multiples of 8; other shapes are refused (YALM_ERR_ARG: use yalm_head_matmul).
+int yalm_head_matmul_mfma(const void* in, int in_dtype, long in_row, int in_head, int in_off, const void* wn, void* out,
+                          int out_dtype, long out_row, int out_head, int out_off, float scale, const float* gate,
+                          long gate_row, int T, int H, int K, int N, hipStream_t stream);
 int yalm_latent_pack(const float* proj, long proj_row, int q_head, int q_rot_off, int kv_off, const void* norm_w,
                      int norm_dtype, float eps, float q_scale, float* out, int T, int H, int rot, int rank, int Dk,
                      int has_kv, hipStream_t stream);

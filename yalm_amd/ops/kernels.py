@@ -765,13 +765,20 @@ def polynorm(z, coef, eps, out):
 HEAD_MATMUL_MAX_K = 512
 
 
-def head_matmul(src, src_head, src_off, wt, out, out_head, out_off, scale=1.0, gate=None):
+HEAD_MATMUL_MFMA_MIN_ROWS = 64
+
+
+def head_matmul(src, src_head, src_off, wt, out, out_head, out_off, scale=1.0, gate=None, wt_nk=None):
     """For every row t and head h: out[t, h * out_head + out_off + n] = scale * sum_k src[t, h * src_head + src_off + k]
     * wt[h, k, n], times sigmoid(gate[t, h * N + n]) if gate (float32 [T, >= H * N]) is given.  src and out are
     2-D, their rows may be wider than the heads they hold; wt [H, K, N].  Types (src, wt, out): all float32;
-    float32, bfloat16, float32; all bfloat16."""
+    float32, bfloat16, float32; all bfloat16.  wt_nk (optional; bfloat16 [H, N, K], wt with its last axes exchanged): with
+    HEAD_MATMUL_MFMA_MIN_ROWS rows or more, and sizes that keep 8 values of a row aligned, the product runs on the matrix
+    cores (the rows rounded to bfloat16)."""
     H, K, N = wt.shape
     T = src.shape[0]
+    mfma = (wt_nk is not None and T >= HEAD_MATMUL_MFMA_MIN_ROWS and not FORCE_SIMPLE and wt_nk.dtype == torch.bfloat16
+            and K % 8 == 0 and src.shape[1] % 8 == 0 and src_head % 8 == 0 and src_off % 8 == 0)
     if K > HEAD_MATMUL_MAX_K:
         raise ValueError("head_matmul: %d inner elements a head, at most %d" % (K, HEAD_MATMUL_MAX_K))
     if src_off + K > src_head or out_off + N > out_head or H * src_head > src.shape[1] or H * out_head > out.shape[1]:
@@ -784,6 +791,12 @@ def head_matmul(src, src_head, src_off, wt, out, out_head, out_off, scale=1.0, g
                 or gate.dtype != torch.float32 or not gate.is_cuda:
             raise ValueError("head_matmul: gate must be float32 [T, >= heads * N] with unit column stride on the GPU")
         p_g = gate.data_ptr()
+    if mfma:
+        library.check(library.lib().yalm_head_matmul_mfma(
+            _need(src, "src", None, (T, None)), dtype_code(src.dtype), src.shape[1], src_head, src_off,
+            _need(wt_nk, "wt_nk", torch.bfloat16, (H, N, K)), _need(out, "out", None, (T, None)), dtype_code(out.dtype),
+            out.shape[1], out_head, out_off, float(scale), p_g, g_row, T, H, K, N, _stream()), "head_matmul on the matrix cores")
+        return out
     library.check(library.lib().yalm_head_matmul(
         _need(src, "src", None, (T, None)), dtype_code(src.dtype), src.shape[1], src_head, src_off,
         _need(wt, "wt"), dtype_code(wt.dtype), _need(out, "out", None, (T, None)), dtype_code(out.dtype), out.shape[1],

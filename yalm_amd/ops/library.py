@@ -53,6 +53,8 @@ _SIGNATURES = {
     "yalm_polynorm": (_I, [_P, _P, _F, _P, _I, _I, _I, _P]),
     "yalm_head_matmul": (_I, [_P, _I, ctypes.c_long, _I, _I, _P, _I, _P, _I, ctypes.c_long, _I, _I, _F, _P, ctypes.c_long,
                               _I, _I, _I, _I, _P]),
+    "yalm_head_matmul_mfma": (_I, [_P, _I, ctypes.c_long, _I, _I, _P, _P, _I, ctypes.c_long, _I, _I, _F, _P, ctypes.c_long,
+                                   _I, _I, _I, _I, _P]),
     "yalm_latent_pack": (_I, [_P, ctypes.c_long, _I, _I, _I, _P, _I, _F, _F, _P, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_moe_route": (_I, [_P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _P]),
     "yalm_moe_select": (_I, [_P, _P, _P, _I, _I, _I, _I, _P]),
@@ -64,7 +66,7 @@ _SIGNATURES = {
     "yalm_probe_mfma": (_I, [_I, _I, _I, _P, _P, _P]),
 }
 
-ABI_VERSION = 27
+ABI_VERSION = 28
 
 
 class KernelError(RuntimeError):

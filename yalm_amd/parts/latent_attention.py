@@ -21,7 +21,8 @@ j with 0 <= i - j < n.  Rotation: the `position` part (pairs (i, i + dims/2) of 
 adjacent at load).
 
 Load-time layout: [W_q; W_dkv; W_g] is one matrix (one product reads h once); W_uk is used as [H, d, R],
-W_uv transposed to [H, R, v]."""
+W_uv transposed to [H, R, v]; with bfloat16 both are kept in the other order too ([H, R, d], [H, v, R]), which the
+matrix-core product of a step of many tokens reads."""
 import math
 
 import torch
@@ -67,7 +68,7 @@ class LatentAttention(Part):
         self.q_cols = self.n_heads * (self.head_dim + self.rot_dim)
         self.kv_cols = self.rank + self.rot_dim if self.own_keys else 0
         self.gate_cols = self.n_heads * self.v_dim if self.gated else 0
-        self.w_in = self.w_uk = self.w_uv = self.w_o = self.kv_norm = None
+        self.w_in = self.w_uk = self.w_uv = self.w_o = self.kv_norm = self.w_uk_nk = self.w_uv_nk = None
 
     def children(self):
         return [self.position]
@@ -108,6 +109,11 @@ class LatentAttention(Part):
         self.w_in = place(torch.cat(blocks, dim=0), compute_dtype, device)
         self.w_uk = place(get(self._name("up_k")).reshape(H, d, R), compute_dtype, device)
         self.w_uv = place(get(self._name("up_v")).reshape(H, self.v_dim, R).transpose(1, 2), compute_dtype, device)
+        # the other order of the same (small) matrices, for the matrix-core product of a step of many tokens
+        self.w_uk_nk = self.w_uv_nk = None
+        if compute_dtype == torch.bfloat16:
+            self.w_uk_nk = self.w_uk.transpose(1, 2).contiguous()
+            self.w_uv_nk = self.w_uv.transpose(1, 2).contiguous()
         self.w_o = place(get(self._name("out")), compute_dtype, device)
 
     def weight_bytes(self):
@@ -157,7 +163,7 @@ class LatentAttention(Part):
         heads = ws.get("latent.heads", (T, (H + 2) * P), torch.float32)
         q_scale = self.scale * math.sqrt(P)
         kernels.latent_pack(proj, d + r, d, self.q_cols, self.kv_norm, self.eps, q_scale, heads, H, r, R, P, self.own_keys)
-        kernels.head_matmul(proj, d + r, 0, self.w_uk, heads, P, r, scale=q_scale)
+        kernels.head_matmul(proj, d + r, 0, self.w_uk, heads, P, r, scale=q_scale, wt_nk=self.w_uk_nk)
         # 3. rotation, cache write, attention over the latent head
         q = ws.get("attn.q", (T, H * P), act)
         group = ctx.cache.group_of(line)
@@ -193,6 +199,6 @@ class LatentAttention(Part):
         # 4. the heads' values from their latent results, the gate, the output projection
         values = ws.get("latent.values", (T, H * self.v_dim), act)
         gate = proj[:, self.q_cols + self.kv_cols:] if self.gated else None
-        kernels.head_matmul(o, P, r, self.w_uv, values, self.v_dim, 0, gate=gate)
+        kernels.head_matmul(o, P, r, self.w_uv, values, self.v_dim, 0, gate=gate, wt_nk=self.w_uv_nk)
         self._gemm(ctx, values, self.w_o, out, epilogue)
         return out
