@@ -28,27 +28,40 @@ __global__ __launch_bounds__(HM_THREADS) void head_matmul_kernel(const TI* __res
   __shared__ float tile[HM_TOK][HM_KMAX];
   const int h = blockIdx.y;
   const int t0 = blockIdx.x * HM_TOK;
+  const int tg = threadIdx.x / WAVE;        // a wave takes 4 of the 16 tokens
+  const int lane = threadIdx.x % WAVE;
+  const TW* w = wt + (size_t)h * K * N;
+  const int n = blockIdx.z * WAVE + lane;          // a workgroup owns 64 columns of the head's result
+  // the first 64 weights of the lane's column are asked for before the tokens' values, so that the two waits are one
+  constexpr int FIRST = 64;
+  TW w0[FIRST];
+#pragma unroll
+  for (int i = 0; i < FIRST; ++i) w0[i] = w[(size_t)min(i, K - 1) * N + min(n, N - 1)];
   for (int i = threadIdx.x; i < HM_TOK * K; i += HM_THREADS) {
     const int tt = i / K, k = i % K;
     const int t = t0 + tt;
     tile[tt][k] = t < T ? to_f32(in[(size_t)t * in_row + (size_t)h * in_head + in_off + k]) : 0.f;
   }
   __syncthreads();
-  const int tg = threadIdx.x / WAVE;        // a wave takes 4 of the 16 tokens
-  const int lane = threadIdx.x % WAVE;
-  const TW* w = wt + (size_t)h * K * N;
-  const int n = blockIdx.z * WAVE + lane;          // a workgroup owns 64 columns of the head's result
   if (n < N) {
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    int k = 0;
-    for (; k + 8 <= K; k += 8) {                     // eight loads in flight, then their products
-      float wv[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) wv[i] = to_f32(w[(size_t)(k + i) * N + n]);
+    for (int i = 0; i < FIRST; ++i) {
+      if (i < K) {                                   // (what lies behind K in the tile was never written)
+        const float wv = to_f32(w0[i]);
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
+        for (int j = 0; j < 4; ++j) acc[j] += tile[tg * 4 + j][i] * wv;
+      }
+    }
+    int k = FIRST;
+    for (; k + 32 <= K; k += 32) {                   // thirty-two loads in flight, then their products
+      TW wv[32];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] += tile[tg * 4 + j][k + i] * wv[i];
+      for (int i = 0; i < 32; ++i) wv[i] = w[(size_t)(k + i) * N + n];
+#pragma unroll
+      for (int i = 0; i < 32; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] += tile[tg * 4 + j][k + i] * to_f32(wv[i]);
     }
     for (; k < K; ++k) {
       const float wv = to_f32(w[(size_t)k * N + n]);
