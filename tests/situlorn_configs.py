@@ -62,7 +62,15 @@ WIDE_LATENT = {"architecture": "Situlorn", "vocab": 128, "width": 64, "norm": {"
                "layers": [layer(mixer(2, 16, 16, 16, 128, 0.1, 10000.0), dense(96)),
                           layer(mixer(2, 16, 16, 16, 128, 0.1, 10000.0, kv_from=0), moe(8, 3, 32, 2.5))]}
 
-ALL = {"mixed": MIXED, "windows": WINDOWS, "only_full": ONLY_FULL, "only_window": ONLY_WINDOW,
+# sizes that are multiples of nothing (no 16-byte loads, no matrix-core products anywhere), one expert, one head, a
+# mixer that rotates nothing
+ODD = {"architecture": "Situlorn", "vocab": 101, "width": 50, "norm": {"eps": 2e-5},
+       "layers": [layer(mixer(3, 6, 2, 5, 10, 0.3, 10000.0), dense(30)),
+                  layer(mixer(1, 7, 0, 9, 13, 0.2, 10000.0), moe(1, 1, 11, 0.5)),
+                  layer(mixer(2, 5, 6, 3, 9, 0.35, 900.0, window=9, scaling=(4.0, 16, 8.0, 1.0)), moe(7, 3, 9, 2.0)),
+                  layer(mixer(2, 3, 2, 7, 10, 0.3, 10000.0, kv_from=0), None)]}
+
+ALL = {"odd": ODD, "mixed": MIXED, "windows": WINDOWS, "only_full": ONLY_FULL, "only_window": ONLY_WINDOW,
        "wide_latent": WIDE_LATENT}
 
 
