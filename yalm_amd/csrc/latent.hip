@@ -32,11 +32,18 @@ __global__ __launch_bounds__(HM_THREADS) void head_matmul_kernel(const TI* __res
   const int lane = threadIdx.x % WAVE;
   const TW* w = wt + (size_t)h * K * N;
   const int n = blockIdx.z * WAVE + lane;          // a workgroup owns 64 columns of the head's result
-  // the first 64 weights of the lane's column are asked for before the tokens' values, so that the two waits are one
-  constexpr int FIRST = 64;
+  // the first 128 weights of the lane's column (all of them, at most sizes) and the gate's values are asked for
+  // before the tokens' values, so that the waits for memory are one
+  constexpr int FIRST = 128;
   TW w0[FIRST];
 #pragma unroll
   for (int i = 0; i < FIRST; ++i) w0[i] = w[(size_t)min(i, K - 1) * N + min(n, N - 1)];
+  float g4[4] = {0.f, 0.f, 0.f, 0.f};
+  if (gate != nullptr) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      g4[j] = gate[(size_t)min(t0 + tg * 4 + j, T - 1) * gate_row + (size_t)h * N + min(n, N - 1)];
+  }
   for (int i = threadIdx.x; i < HM_TOK * K; i += HM_THREADS) {
     const int tt = i / K, k = i % K;
     const int t = t0 + tt;
@@ -73,10 +80,7 @@ __global__ __launch_bounds__(HM_THREADS) void head_matmul_kernel(const TI* __res
       const int t = t0 + tg * 4 + j;
       if (t >= T) continue;
       float v = acc[j] * scale;
-      if (gate != nullptr) {
-        const float g = gate[(size_t)t * gate_row + (size_t)h * N + n];
-        v *= 1.0f / (1.0f + expf(-g));
-      }
+      if (gate != nullptr) v *= 1.0f / (1.0f + expf(-g4[j]));
       out[(size_t)t * out_row + (size_t)h * out_head + out_off + n] = from_f32<TO>(v);
     }
   }

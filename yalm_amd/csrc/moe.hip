@@ -125,11 +125,20 @@ __global__ __launch_bounds__(PAIR_WAVES * WAVE) void moe_pair_down_kernel(const 
   const int d0 = blockIdx.y * PAIR_ROWS;
   for (int d = d0 + wave; d < min(D, d0 + PAIR_ROWS); d += PAIR_WAVES) {
     float acc = 0.f;
-    for (int k = 0; k < top; ++k) {
-      const int e = ids[(size_t)t * top + k];
-      if (e < 0 || e >= E) continue;
-      const float v = wave_sum(dot_row<T>(w_down + ((size_t)e * D + d) * F, mid + ((size_t)t * top + k) * F, F, lane));
-      acc += wts[(size_t)t * top + k] * v;
+    for (int k0 = 0; k0 < top; k0 += 4) {          // four choices' rows at a time: their loads are in flight together
+      float part[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int k = k0 + i;
+        const int e = k < top ? ids[(size_t)t * top + k] : -1;
+        part[i] = e >= 0 && e < E ? dot_row<T>(w_down + ((size_t)e * D + d) * F, mid + ((size_t)t * top + k) * F, F, lane) : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int k = k0 + i;
+        const float v = wave_sum(part[i]);
+        if (k < top) acc += wts[(size_t)t * top + k] * v;    // in the order of the choices
+      }
     }
     if (lane == 0) out[(size_t)t * D + d] = accumulate ? out[(size_t)t * D + d] + acc : acc;
   }
