@@ -70,7 +70,13 @@ ODD = {"architecture": "Situlorn", "vocab": 101, "width": 50, "norm": {"eps": 2e
                   layer(mixer(2, 5, 6, 3, 9, 0.35, 900.0, window=9, scaling=(4.0, 16, 8.0, 1.0)), moe(7, 3, 9, 2.0)),
                   layer(mixer(2, 3, 2, 7, 10, 0.3, 10000.0, kv_from=0), None)]}
 
-ALL = {"odd": ODD, "mixed": MIXED, "windows": WINDOWS, "only_full": ONLY_FULL, "only_window": ONLY_WINDOW,
+# a latent head of 336 (320 + 16): beyond 256 a lane of the float32-arithmetic attention holds 16 elements, not 4
+HUGE_LATENT = {"architecture": "Situlorn", "vocab": 96, "width": 64, "norm": {"eps": 1e-5},
+               "layers": [layer(mixer(2, 16, 16, 24, 320, 0.05, 10000.0), dense(64)),
+                          layer(mixer(3, 8, 16, 16, 320, 0.05, 10000.0, kv_from=0), None),
+                          layer(mixer(2, 16, 8, 24, 300, 0.05, 10000.0, window=33, scaling=(4.0, 64, 16.0, 1.0)), dense(48))]}
+
+ALL = {"huge_latent": HUGE_LATENT, "odd": ODD, "mixed": MIXED, "windows": WINDOWS, "only_full": ONLY_FULL, "only_window": ONLY_WINDOW,
        "wide_latent": WIDE_LATENT}
 
 

@@ -358,9 +358,10 @@ def compare(folders, name, dtype, steps, requests, engine, what):
         assert g.pool.n_free == g.n_pages
 
 
-LENGTHS = {"odd": [1, 9, 10, 70, 129], "mixed": [1, 2, 23, 64, 65, 150, 330], "windows": [1, 5, 6, 64, 66, 131, 200, 340],
+LENGTHS = {"huge_latent": [1, 40, 131], "odd": [1, 9, 10, 70, 129], "mixed": [1, 2, 23, 64, 65, 150, 330], "windows": [1, 5, 6, 64, 66, 131, 200, 340],
            "only_full": [3, 70], "only_window": [3, 7, 8, 70], "wide_latent": [2, 100, 350]}
-GROUPS = {"odd": [([0, 1, 2, 3], [1, 3, 10, 64]), ([4, 3], [100, 1])],
+GROUPS = {"huge_latent": [([0, 1, 2], [1, 20, 100])],
+          "odd": [([0, 1, 2, 3], [1, 3, 10, 64]), ([4, 3], [100, 1])],
           "mixed": [([0, 2, 4, 5], [1, 23, 60, 100]), ([6, 1, 3], [321, 2, 64]), ([5, 4], [2, 1])],
           "windows": [([0, 1, 2, 3], [1, 5, 2, 64]), ([4, 5, 6], [63, 100, 130]), ([7, 6], [330, 1])],
           "only_full": [([0, 1], [1, 40])], "only_window": [([0, 1, 2, 3], [2, 1, 8, 30])],

@@ -31,20 +31,22 @@ struct ScoreBias {
   }
 };
 
-constexpr int MAX_HD = 256;              // head sizes up to 256 (4 output elements per lane)
-constexpr int ACC = MAX_HD / WAVE;
+// A lane holds ACC output elements: 4 for head sizes up to 256 (every model with heads of its own), 16 for heads up
+// to 1,024 (a latent attention's one wide head); the kernels are compiled for both.
+constexpr int MAX_HD = 1024;
+constexpr int ACC_SMALL = 4, ACC_BIG = MAX_HD / WAVE;
 constexpr int COMBINE_THREADS = 256;
 
 // ---------------------------------------------------------------------------
 // prefill: a step's tokens over the same step's keys
 // ---------------------------------------------------------------------------
-template <typename T>
+template <typename T, int ACC>
 __global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
     const T* __restrict__ q, const T* __restrict__ k_stage, const T* __restrict__ v_stage, T* __restrict__ out,
     float* __restrict__ out_f32, float* __restrict__ lse, const int* __restrict__ seq_tile0,
     const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int n_heads, int n_kv_heads, int hd, int window,
     ScoreBias sb) {
-  __shared__ float qs[MAX_HD];
+  __shared__ float qs[ACC * WAVE];
   __shared__ float ps[WAVE];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int b = tok_seq[t], pos = tok_pos[t];
@@ -111,13 +113,13 @@ __global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
 // decode: one query per sequence over the pages of the cache, split over pages
 // partial layout: [B, n_heads, n_splits, hd + 2] = (acc[hd], m, l)
 // ---------------------------------------------------------------------------
-template <typename T>
+template <typename T, int ACC>
 __global__ __launch_bounds__(WAVE) void attn_decode_simple_kernel(
     const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_len, float* __restrict__ partial, int n_heads, int n_kv_heads, int hd, int window,
     int n_splits, int n_pages, int page_layout, ScoreBias sb) {
-  __shared__ float qs[MAX_HD];
+  __shared__ float qs[ACC * WAVE];
   __shared__ float ps[WAVE];
   const int b = blockIdx.x, h = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
   float* part = partial + (((size_t)b * n_heads + h) * n_splits + split) * (hd + 2);
@@ -191,7 +193,7 @@ __global__ __launch_bounds__(WAVE) void attn_decode_simple_kernel(
 // here, with the keys turned, while the splits' loads are in flight; and a token at one of its
 // sequence's first positions stores its key and value as a sink (no query of the launch reads it: one
 // token a sequence, and the window, at least n_sinks wide, still covers it).
-template <typename T, bool BASE2 = false>
+template <typename T, bool BASE2 = false, int ACC = ACC_SMALL>
 __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(const float* __restrict__ partial,
                                                                              T* __restrict__ out,
                                                                              float* __restrict__ lse, int n_heads,
@@ -201,7 +203,7 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(co
   // splits of the weighted sum and add their parts in a fixed order).
   constexpr int NWV = COMBINE_THREADS / WAVE;
   constexpr int PRE = 4;                          // splits a wave asks for ahead
-  __shared__ float accs[NWV][MAX_HD];
+  __shared__ float accs[NWV][ACC * WAVE];
   const int b = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x & (WAVE - 1), g = threadIdx.x / WAVE;
   const int stride = hd + 2;
@@ -319,10 +321,14 @@ extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const v
   const ScoreBias sb = {score_bias, n_bias};
   dim3 grid(T, n_heads);
   if (dtype == YALM_F32) {
-    attn_prefill_simple_kernel<float><<<grid, WAVE, 0, stream>>>((const float*)q, (const float*)k_stage,
-                                                                 (const float*)v_stage, (float*)out, out_f32, lse, seq_tile0,
-                                                                 tok_seq, tok_pos, n_heads, n_kv_heads, head_dim,
-                                                                 window, sb);
+    if (head_dim <= ACC_SMALL * WAVE)
+      attn_prefill_simple_kernel<float, ACC_SMALL><<<grid, WAVE, 0, stream>>>(
+          (const float*)q, (const float*)k_stage, (const float*)v_stage, (float*)out, out_f32, lse, seq_tile0, tok_seq,
+          tok_pos, n_heads, n_kv_heads, head_dim, window, sb);
+    else
+      attn_prefill_simple_kernel<float, ACC_BIG><<<grid, WAVE, 0, stream>>>(
+          (const float*)q, (const float*)k_stage, (const float*)v_stage, (float*)out, out_f32, lse, seq_tile0, tok_seq,
+          tok_pos, n_heads, n_kv_heads, head_dim, window, sb);
     return launch_status();
   }
   if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
@@ -331,9 +337,14 @@ extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const v
                                          n_tiles, n_heads, n_kv_heads, head_dim, window, score_bias, n_bias, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
-  attn_prefill_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>((const bf16*)q, (const bf16*)k_stage,
-                                                              (const bf16*)v_stage, (bf16*)out, out_f32, lse, seq_tile0, tok_seq,
-                                                              tok_pos, n_heads, n_kv_heads, head_dim, window, sb);
+  if (head_dim <= ACC_SMALL * WAVE)
+    attn_prefill_simple_kernel<bf16, ACC_SMALL><<<grid, WAVE, 0, stream>>>(
+        (const bf16*)q, (const bf16*)k_stage, (const bf16*)v_stage, (bf16*)out, out_f32, lse, seq_tile0, tok_seq, tok_pos,
+        n_heads, n_kv_heads, head_dim, window, sb);
+  else
+    attn_prefill_simple_kernel<bf16, ACC_BIG><<<grid, WAVE, 0, stream>>>(
+        (const bf16*)q, (const bf16*)k_stage, (const bf16*)v_stage, (bf16*)out, out_f32, lse, seq_tile0, tok_seq, tok_pos,
+        n_heads, n_kv_heads, head_dim, window, sb);
   return launch_status();
 }
 
@@ -378,11 +389,19 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
     return YALM_ERR_ARG;
   dim3 grid(B, n_heads, n_splits), cgrid(B, n_heads);
   if (dtype == YALM_F32) {
-    attn_decode_simple_kernel<float><<<grid, WAVE, 0, stream>>>(
-        (const float*)q, (const float*)k_pages, (const float*)v_pages, block_table, table_stride, ring_pages,
-        seq_slot, seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, sb);
-    attn_decode_combine_kernel<float><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (float*)out, lse, n_heads,
-                                                                             head_dim, n_splits, sinks);
+    if (head_dim <= ACC_SMALL * WAVE) {
+      attn_decode_simple_kernel<float, ACC_SMALL><<<grid, WAVE, 0, stream>>>(
+          (const float*)q, (const float*)k_pages, (const float*)v_pages, block_table, table_stride, ring_pages,
+          seq_slot, seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, sb);
+      attn_decode_combine_kernel<float><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (float*)out, lse, n_heads,
+                                                                               head_dim, n_splits, sinks);
+    } else {
+      attn_decode_simple_kernel<float, ACC_BIG><<<grid, WAVE, 0, stream>>>(
+          (const float*)q, (const float*)k_pages, (const float*)v_pages, block_table, table_stride, ring_pages,
+          seq_slot, seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, sb);
+      attn_decode_combine_kernel<float, false, ACC_BIG><<<cgrid, COMBINE_THREADS, 0, stream>>>(
+          partial, (float*)out, lse, n_heads, head_dim, n_splits, sinks);
+    }
     return launch_status();
   }
   if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
@@ -392,11 +411,19 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
                                         n_pages, page_layout, sinks, step_max_len, seq_order, score_bias, n_bias, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
-  attn_decode_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>(
-      (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot,
-      seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, sb);
-  attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads, head_dim,
-                                                                          n_splits, sinks);
+  if (head_dim <= ACC_SMALL * WAVE) {
+    attn_decode_simple_kernel<bf16, ACC_SMALL><<<grid, WAVE, 0, stream>>>(
+        (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot,
+        seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, sb);
+    attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads, head_dim,
+                                                                            n_splits, sinks);
+  } else {
+    attn_decode_simple_kernel<bf16, ACC_BIG><<<grid, WAVE, 0, stream>>>(
+        (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot,
+        seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, sb);
+    attn_decode_combine_kernel<bf16, false, ACC_BIG><<<cgrid, COMBINE_THREADS, 0, stream>>>(
+        partial, (bf16*)out, lse, n_heads, head_dim, n_splits, sinks);
+  }
   return launch_status();
 }
 }  // namespace

@@ -13,7 +13,7 @@ from . import library
 
 PAGE = 64                       # tokens per cache page (csrc/common.h)
 PREFILL_MIXED_TILES = 64        # prefill_tile_order mixes the sequences of a step up to this many tiles
-MAX_HEAD_DIM = 256
+MAX_HEAD_DIM = 1024             # of the float32-arithmetic attention kernels (above 256: a latent attention's one wide head)
 MFMA_HEAD_DIMS = tuple(range(16, 129, 16))   # head sizes of the matrix-core attention kernels (others: float32 arithmetic)
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
