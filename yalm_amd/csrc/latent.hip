@@ -44,20 +44,26 @@ __global__ __launch_bounds__(HM_THREADS) void head_matmul_kernel(const TI* __res
     for (int j = 0; j < 4; ++j)
       g4[j] = gate[(size_t)min(t0 + tg * 4 + j, T - 1) * gate_row + (size_t)h * N + min(n, N - 1)];
   }
-  for (int i = threadIdx.x; i < HM_TOK * K; i += HM_THREADS) {
-    const int tt = i / K, k = i % K;
+  const int Kt = max(K, FIRST);                    // the tile is filled to FIRST columns at least, zeros behind K
+  for (int i = threadIdx.x; i < HM_TOK * Kt; i += HM_THREADS) {
+    const int tt = i / Kt, k = i % Kt;
     const int t = t0 + tt;
-    tile[tt][k] = t < T ? to_f32(in[(size_t)t * in_row + (size_t)h * in_head + in_off + k]) : 0.f;
+    tile[tt][k] = t < T && k < K ? to_f32(in[(size_t)t * in_row + (size_t)h * in_head + in_off + k]) : 0.f;
   }
   __syncthreads();
   if (n < N) {
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    // no branch in these 128 steps (behind K the tile holds zeros and the weights count as zero), so that the
+    // reads of the tile run ahead of the products
 #pragma unroll
-    for (int i = 0; i < FIRST; ++i) {
-      if (i < K) {                                   // (what lies behind K in the tile was never written)
-        const float wv = to_f32(w0[i]);
+    for (int i0 = 0; i0 < FIRST; i0 += 4) {
+      float wv[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] += tile[tg * 4 + j][i] * wv;
+      for (int i = 0; i < 4; ++i) wv[i] = i0 + i < K ? to_f32(w0[i0 + i]) : 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float4 a = *reinterpret_cast<const float4*>(&tile[tg * 4 + j][i0]);
+        acc[j] += a.x * wv[0] + a.y * wv[1] + a.z * wv[2] + a.w * wv[3];
       }
     }
     int k = FIRST;
