@@ -130,3 +130,23 @@ def test_plain_window_of_one_sees_only_itself():
     v = c @ w["l0.mix.uv"].T
     want = (v * torch.sigmoid(h @ w["l0.mix.g"].T)) @ w["l0.mix.o"].T
     assert torch.allclose(out, want, rtol=1e-12, atol=1e-12)
+
+
+def test_the_measured_configurations_are_valid():
+    """bench.py --design situlorn builds these; they pass the configuration's checks and their Llama
+    counterparts have about as many dense weights."""
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+    from yalm_amd.config import config_from_dict
+    from yalm_amd.engine.model import param_specs_of
+    for width in (2048, 4096):
+        cfg = config_from_dict(bench.situlorn_config(width))
+        spec = cfg.to_spec()
+        assert [e.writes_cache for e in spec.schedule] == [True, False, True, True]
+        sizes = {s.name: 1 for s in param_specs_of(spec)}
+        assert "l1.mix.dkv" not in sizes and "l0.mix.dkv" in sizes and "l2.mix.g" in sizes
+        llama = config_from_dict(bench.llama_config(width))
+        dense = 2 * width * bench.situlorn_config(width)["layers"][0]["mlp"]["ff"]
+        assert abs(dense - 3 * width * llama.intermediate_size) <= 0.01 * dense
