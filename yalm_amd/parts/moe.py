@@ -8,10 +8,10 @@ a token's chosen experts, in the order of their scores.
 
 The experts' matrices are stacked at load ([E, F, D], [E, F, D], [E, D, F]); routing happens on the device
 (nothing of it reaches the host, so a decode step stays a captured graph), and every (token, choice) pair is
-served from its expert's weights.  A step of whole prompts with GROUPED_MIN_TOKENS tokens or more (bfloat16) groups
-the pairs by expert instead and multiplies every expert's rows as tiles on the matrix cores, all experts in one
-launch a product; so does a decode step of GROUPED_MIN_DECODE_ROWS rows or more, where the grouped products read
-every chosen expert once while the pairs would read it once a pair (measured at width 4,096, 32 experts of 2,048,
+served from its expert's weights.  A step of GROUPED_MIN_ROWS rows or more (bfloat16; whole prompts, and decode
+batches of 16 and more) groups the pairs by expert instead and multiplies every expert's rows as tiles on the
+matrix cores, all experts in one launch a product: the grouped products read every chosen expert once while the
+pairs would read it once a pair (measured at width 4,096, 32 experts of 2,048,
 4 a token, four layers: batch 8 1.01 against 1.03 ms a step, batch 16 1.46 against 1.15, batch 64 3.32 against 1.44,
 batch 128 5.54 against 1.60).  Both ways are decided on the device, so a decode step stays a captured graph."""
 import torch
@@ -21,8 +21,7 @@ from ..weights.loader import ParamSpec, place
 from .base import Part, part
 
 
-GROUPED_MIN_TOKENS = 48          # whole prompts: from this many tokens on the pairs are grouped by expert
-GROUPED_MIN_DECODE_ROWS = 9      # decode steps: from this many rows on (batches of 16 rows and more)
+GROUPED_MIN_ROWS = 9             # steps of this many rows and more group the pairs by expert
 
 
 @part("feed_forward", "moe")
@@ -78,8 +77,7 @@ class MixtureOfExperts(Part):
         logits = ws.get("moe.logits", (T, self.n_experts), torch.float32)        # products exact, sums in float32
         self._gemm(ctx, h, self.w_router, logits, kernels.EPI_STORE_F32)
         kernels.moe_select(logits, ids, wts, self.renormalize)
-        if T >= (GROUPED_MIN_TOKENS if ctx.mode == "prefill" else GROUPED_MIN_DECODE_ROWS) \
-                and kernels.can_moe_grouped(self.dim, self.hidden, h.dtype):
+        if T >= GROUPED_MIN_ROWS and kernels.can_moe_grouped(self.dim, self.hidden, h.dtype):
             return kernels.moe_grouped(h, self.w_gate, self.w_up, self.w_down, ids, wts, self.limit, self.alpha, ws.get,
                                        out, accumulate)
         mid = ws.get("moe.hidden", (T * self.top, self.hidden), h.dtype)
