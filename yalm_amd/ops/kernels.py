@@ -881,9 +881,10 @@ def moe_pair_down(mid, w_down, ids, wts, out, accumulate=False):
 MOE_GROUP_ROWS = 128           # rows of a tile of the grouped products (csrc/moe.hip)
 
 
-def can_moe_grouped(D, F, dtype):
-    """Whether moe_grouped takes these sizes."""
-    return dtype == torch.bfloat16 and D % 8 == 0 and F % 8 == 0 and not FORCE_SIMPLE
+def can_moe_grouped(D, F, dtype, n_pairs=0, n_experts=0):
+    """Whether moe_grouped takes these sizes (and this many pairs: its tiles are one axis of a launch)."""
+    return dtype == torch.bfloat16 and D % 8 == 0 and F % 8 == 0 and not FORCE_SIMPLE \
+        and (n_pairs + MOE_GROUP_ROWS - 1) // MOE_GROUP_ROWS + n_experts <= 65535
 
 
 def moe_grouped_tiles(n_pairs, n_experts):

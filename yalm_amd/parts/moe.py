@@ -77,7 +77,7 @@ class MixtureOfExperts(Part):
         logits = ws.get("moe.logits", (T, self.n_experts), torch.float32)        # products exact, sums in float32
         self._gemm(ctx, h, self.w_router, logits, kernels.EPI_STORE_F32)
         kernels.moe_select(logits, ids, wts, self.renormalize)
-        if T >= GROUPED_MIN_ROWS and kernels.can_moe_grouped(self.dim, self.hidden, h.dtype):
+        if T >= GROUPED_MIN_ROWS and kernels.can_moe_grouped(self.dim, self.hidden, h.dtype, T * self.top, self.n_experts):
             return kernels.moe_grouped(h, self.w_gate, self.w_up, self.w_down, ids, wts, self.limit, self.alpha, ws.get,
                                        out, accumulate)
         mid = ws.get("moe.hidden", (T * self.top, self.hidden), h.dtype)
