@@ -33,7 +33,7 @@ def randn(*shape, seed=0, scale=1.0):
 
 
 # ------------------------------------------------------------------------------------------ kernels alone
-@pytest.mark.parametrize("R_,D", [(1, 8), (5, 80), (33, 1000), (3, 4097)])
+@pytest.mark.parametrize("R_,D", [(1, 8), (5, 80), (33, 1000), (3, 4097), (2, 9001)])
 @pytest.mark.parametrize("out_dtype", [None, torch.bfloat16, torch.float32])
 def test_norm_add(R_, D, out_dtype):
     from yalm_amd.ops import kernels
@@ -58,7 +58,7 @@ def test_norm_add(R_, D, out_dtype):
     assert torch.allclose(xd.cpu().to(F64), x.to(F64) + P.rms_norm(y.to(F64), wb.to(F64), 1e-5), rtol=1e-5, atol=1e-5)
 
 
-@pytest.mark.parametrize("R_,F", [(1, 4), (7, 112), (20, 1500)])
+@pytest.mark.parametrize("R_,F", [(1, 4), (7, 112), (20, 1500), (3, 8200), (2, 40001)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_polynorm(R_, F, out_dtype):
     from yalm_amd.ops import kernels
@@ -525,6 +525,20 @@ def test_greedy_generation_and_command_line(folders):
     assert p.returncode == 0, p.stderr[-3000:]
     printed = p.stdout.split("\n\n")[0].split("\n", 1)[1].split()
     assert [int(t) for t in printed] == out[0]
+
+
+def test_token_probabilities(folders):
+    """The step function's other result, the probability of a given next token at every place (what the command
+    line's perplexity mode uses), against the plain logits' softmax."""
+    name = "mixed"
+    engine = engine_for(folders, name, "float32")
+    toks = requests_for(SC.ALL[name], [90], seed=14)["r0"]
+    slots = engine.start(1)
+    probs = engine.step(slots, [toks], [list(range(len(toks) - 1))], targets=[toks[1:]]).cpu().numpy()
+    engine.release(slots)
+    want = torch.softmax(torch.from_numpy(plain_logits(folders, name, "float32", toks)).double(), dim=-1)
+    want = want[torch.arange(len(toks) - 1), torch.tensor(toks[1:])].numpy()
+    assert np.allclose(probs, want, rtol=2e-3, atol=1e-6)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
