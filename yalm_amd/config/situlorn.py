@@ -22,7 +22,7 @@ from .spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
 
 MIXERS = ("latent_attention", "latent_attention_2")
 EXPERT_ALPHA = 1.702             # g sigmoid(alpha g) in the experts
-POSITIONS = 1 << 20              # the design names no longest sequence: the engine's cache bounds it
+POSITIONS = 1 << 18              # the design names no longest sequence: the cache bounds it (and this, where every layer keeps a window)
 
 
 def _need(d, key, where):
