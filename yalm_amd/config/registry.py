@@ -6,6 +6,7 @@ import json
 import os
 
 from .llama import ConfigError, LlamaConfig
+from .gedunex import GedunexConfig
 from .situlorn import SitulornConfig
 
 _ARCHITECTURES = {}
@@ -43,6 +44,6 @@ def config_from_folder(path):
         return config_from_dict(json.load(fh))
 
 
-for _cls in (LlamaConfig, SitulornConfig):
+for _cls in (LlamaConfig, SitulornConfig, GedunexConfig):
     for _name in _cls.ARCHITECTURES:
         register_architecture(_name, _cls)

@@ -4,7 +4,8 @@
 
 // attention_simple.hip; base2: the partial results' maxima are exponents of 2, not of e
 int yalm_attn_decode_combine_bf16(const float* partial, void* out, float* lse, int B, int n_heads, int head_dim,
-                                  int n_splits, int base2, const SinkArgs& sinks, hipStream_t stream);
+                                  int n_splits, int base2, const SinkArgs& sinks, const float* sink_logit,
+                                  hipStream_t stream);
 
 namespace {
 
@@ -17,14 +18,17 @@ namespace {
 // BLOCKS: the pages are laid out in blocks (YALM_PAGE_BLOCKS): every load instruction reads 1 KB of consecutive
 // bytes, and asks for them non-temporally (a step reads a page once; with pieces of lines the hint costs more
 // than it gains: the other half of a line would be fetched again).
-// BIAS: a term is added to every score by the distance of query and key, bias[head][min(distance, n_bias - 1)].
+// BIAS: the scores are shaped (ScoreShape: a cap, a term by the distance of query and key, bias[head][min(distance,
+// n_bias - 1)], a learned logit in the denominator; each optional).
 template <int HD, int NW, bool BLOCKS, bool BIAS>
 __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_kernel(   // 2 waves a SIMD: head size 128 needs their registers
     const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_len, float* __restrict__ partial, bf16* __restrict__ out, float* __restrict__ lse,
     int n_heads, int n_kv_heads, int window, int n_splits, int n_pages, const int* __restrict__ step_max_len,
-    const int* __restrict__ seq_order, const float* __restrict__ bias, int n_bias) {
+    const int* __restrict__ seq_order, ScoreShape shape) {
+  const float* __restrict__ bias = shape.bias;
+  const int n_bias = shape.n_bias;
   // A head size that is no multiple of 32 (pages in rows then): the last step of the scores' product is half empty.
   // The query's lanes of that half hold zeros; the keys' lanes read the row's last 8 elements again (an address
   // inside the row, finite values for every row that counts).
@@ -79,7 +83,7 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
         qv[ks] = head_ok && ks * 32 + qd * 8 < HD ? ld8(qrow + ks * 32 + qd * 8) : zero8();
     }
 
-    const float* bias_row = BIAS ? bias + (size_t)(h0 + min(j, G - 1)) * n_bias : nullptr;   // the column's head
+    const float* bias_row = BIAS && bias != nullptr ? bias + (size_t)(h0 + min(j, G - 1)) * n_bias : nullptr;   // the column's head
     bf16x8 kreg[4][KS];
     auto page_of = [&](int a) { return min(max(table[a % ring_pages], 0), n_pages - 1); };
     auto load_keys = [&](int phys) {
@@ -133,7 +137,9 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
           float v = sc[t][r] * score_scale;
           if constexpr (BIAS) {                    // in the same units as the scores: exponents of 2
             const int dist = L - 1 - (base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r);
-            v = fmaf(bias_row[min(max(dist, 0), n_bias - 1)], 1.4426950408889634f, v);
+            if (shape.softcap > 0.f)                // capped in natural units, then back into exponents of 2
+              v = soft_cap_fast(v * LN2, shape.softcap) * 1.4426950408889634f;
+            if (bias_row != nullptr) v = fmaf(bias_row[min(max(dist, 0), n_bias - 1)], 1.4426950408889634f, v);
           }
           if (edge) {
             int pos = base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r;
@@ -199,7 +205,14 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
     for (int w = 1; w < NW; ++w) lt += sm_l[w][j];
     if (n_splits == 1 && out != nullptr) {        // nothing to merge with: this is the result
       bf16* orow = out + ((size_t)b * n_heads + h0 + j) * HD;
-      const float inv_l = lt > 0.f ? 1.0f / lt : 0.f;
+      float keep = 1.0f;
+      if (BIAS && shape.sink_logit != nullptr && lt > 0.f) {     // the learned logit: in the denominator only
+        const float sk = shape.sink_logit[h0 + j] * 1.4426950408889634f, m_new = fmaxf(m_all, sk);
+        keep = __builtin_amdgcn_exp2f(m_all - m_new);
+        lt = lt * keep + __builtin_amdgcn_exp2f(sk - m_new);
+        m_all = m_new;
+      }
+      const float inv_l = lt > 0.f ? keep / lt : 0.f;
       for (int dt = wave; dt < DT; dt += NW) {
         f32x4 v = sm_o[0][dt][lane];
 #pragma unroll
@@ -232,14 +245,18 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                                float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
                                int n_splits, int n_pages, int page_layout, const SinkArgs& sinks,
-                               const int* step_max_len, const int* seq_order, const float* bias, int n_bias,
+                               const int* step_max_len, const int* seq_order, const ScoreShape& shape,
                                hipStream_t stream) {
+  const float* bias = shape.bias;
+  const int n_bias = shape.n_bias;
+  const bool shaped = shape.any();
   // with sinks the merge kernel always runs: it takes them in, also where there is one split
   const bool merge = n_splits > 1 || sinks.n_sinks > 0;
   if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim)) return YALM_ERR_ARG;
   // a score bias: the engine's layout of the pages only (blocks where the head size allows), and no sinks (they are
   // scored without it)
-  if (bias != nullptr && (n_bias <= 0 || (page_layout != YALM_PAGE_BLOCKS && head_dim % 32 == 0) || sinks.n_sinks > 0))
+  if ((bias != nullptr && n_bias <= 0) ||
+      (shaped && ((page_layout != YALM_PAGE_BLOCKS && head_dim % 32 == 0) || sinks.n_sinks > 0)))
     return YALM_ERR_ARG;
   const int parts_g = (n_heads / n_kv_heads + 15) / 16;      // workgroups a KV head: 16 query heads each
   if ((long)n_kv_heads * parts_g > 65535) return YALM_ERR_ARG;
@@ -248,7 +265,7 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
   attn_decode_mfma_kernel<HD_, NW_, BLOCKS_, BIAS_><<<grid, NW_ * WAVE, 0, stream>>>(                               \
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot, \
       seq_len, partial, merge ? nullptr : (bf16*)out, lse, n_heads, n_kv_heads, window, n_splits, n_pages, \
-      step_max_len, seq_order, bias, n_bias)
+      step_max_len, seq_order, shape)
   // 4 waves a workgroup: 8 measured no faster with one split and slower with more (a CU draws about
   // 33 GB/s whatever its number of waves, so a small batch needs its workgroups spread over all CUs)
   // pages in blocks for the head sizes that are multiples of 32, in rows for the others (and for yalm_attn_decode)
@@ -256,13 +273,13 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
   if (blocks && head_dim % 32 != 0) return YALM_ERR_ARG;
 #define YALM_DECODE_HD32(HD_)                                                       \
   case HD_:                                                                         \
-    if (bias != nullptr) YALM_DECODE(HD_, 4, true, true);                           \
+    if (shaped) YALM_DECODE(HD_, 4, true, true);                                 \
     else if (blocks) YALM_DECODE(HD_, 4, true, false);                              \
     else YALM_DECODE(HD_, 4, false, false);                                         \
     break
 #define YALM_DECODE_HD16(HD_)                                                       \
   case HD_:                                                                         \
-    if (bias != nullptr) YALM_DECODE(HD_, 4, false, true);                          \
+    if (shaped) YALM_DECODE(HD_, 4, false, true);                                \
     else YALM_DECODE(HD_, 4, false, false);                                         \
     break
   switch (head_dim) {
@@ -280,5 +297,5 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
 #undef YALM_DECODE
   int rc = launch_status();
   if (rc != YALM_OK || !merge) return rc;          // one split writes the result itself
-  return yalm_attn_decode_combine_bf16(partial, out, lse, B, n_heads, head_dim, n_splits, 1, sinks, stream);
+  return yalm_attn_decode_combine_bf16(partial, out, lse, B, n_heads, head_dim, n_splits, 1, sinks, shape.sink_logit, stream);
 }

@@ -22,13 +22,16 @@ namespace {
 // compute unit alone and is done in half the time, so that the compute units are no longer held by
 // the few workgroups that see the most keys (with KSPL = 1 the launch lasts as long as its longest
 // workgroup, 32 key tiles at 2,048 tokens, while the mean is 17).
-// BIAS: a term is added to every score by the distance of query and key, bias[head][min(distance, n_bias - 1)].
+// BIAS: the scores are shaped (ScoreShape: a cap, a term by the distance of query and key, bias[head][min(distance,
+// n_bias - 1)], a learned logit in the denominator; each optional).
 template <int HD, int NC, int KSPL, bool BIAS>
 __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_stage, const bf16* __restrict__ v_stage,
     bf16* __restrict__ out, float* __restrict__ out_f32, float* __restrict__ lse, const int* __restrict__ cu_seqlens,
     const int* __restrict__ seq_tile0, const int* __restrict__ tile_order, int fold_at, int B, int n_heads,
-    int n_kv_heads, int window, const float* __restrict__ bias, int n_bias) {
+    int n_kv_heads, int window, ScoreShape shape) {
+  const float* __restrict__ bias = shape.bias;
+  const int n_bias = shape.n_bias;
   // A head size that is no multiple of 32: the last step of the scores' product is half empty (zeros in the query's
   // lanes, the row's last 8 elements once more in the keys'), and the tile's chunks do not divide evenly over the threads.
   constexpr int KS = (HD + 31) / 32, DT = HD / 16;
@@ -70,7 +73,7 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
   const int start = cu_seqlens[b], len = cu_seqlens[b + 1] - start;
   const int g = h / (n_heads / n_kv_heads);
   const float score_scale = 1.4426950408889634f / sqrtf((float)HD);   // log2(e) / sqrt(head_dim)
-  const float* bias_row = BIAS ? bias + (size_t)h * n_bias : nullptr;
+  const float* bias_row = BIAS && bias != nullptr ? bias + (size_t)h * n_bias : nullptr;
 
   const int blk0 = tq * PAGE;                     // first position of the workgroup
   const int pos0 = blk0 + wave * 16 * NC;         // first position of the wave
@@ -179,7 +182,11 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
               float v = sc[c][t][r];
               if constexpr (BIAS) {               // scaled here, with the distance's term in the same units (exponents of 2)
                 const int dist = pos_q[c] - (base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r);
-                v = fmaf(v, score_scale, bias_row[min(max(dist, 0), n_bias - 1)] * 1.4426950408889634f);
+                const float term = bias_row != nullptr ? bias_row[min(max(dist, 0), n_bias - 1)] * 1.4426950408889634f : 0.f;
+                if (shape.softcap > 0.f)           // capped in natural units, then into exponents of 2
+                  v = fmaf(soft_cap_fast(v * (score_scale * LN2), shape.softcap), 1.4426950408889634f, term);
+                else
+                  v = fmaf(v, score_scale, term);
                 sc[c][t][r] = v;
               }
               if (decltype(masked)::value) {
@@ -273,9 +280,16 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
     float lt = l[c];
     lt += __shfl_xor(lt, 16, WAVE);
     lt += __shfl_xor(lt, 32, WAVE);
+    float keep = 1.0f;
+    if (BIAS && shape.sink_logit != nullptr) {    // the learned logit: in the denominator only
+      const float sk = shape.sink_logit[h] * 1.4426950408889634f, m_new = fmaxf(m[c], sk);
+      keep = __builtin_amdgcn_exp2f(m[c] - m_new);
+      lt = lt * keep + __builtin_amdgcn_exp2f(sk - m_new);
+      m[c] = m_new;
+    }
     if (q_ok[c]) {
       bf16* orow = out + ((size_t)(start + pos_q[c]) * n_heads + h) * HD;
-      const float inv_l = 1.0f / lt;
+      const float inv_l = keep / lt;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -310,14 +324,14 @@ template <int HD, int NC, int KSPL, bool BIAS>
 int launch_prefill(dim3 grid, int threads, size_t lds, hipStream_t stream, const bf16* qp, const bf16* kp, const bf16* vp,
                    bf16* out, float* out_f32, float* lse, const int* cu_seqlens, const int* seq_tile0,
                    const int* tile_order, int fold_at, int B, int n_heads, int n_kv_heads, int window,
-                   const float* bias, int n_bias) {
+                   const ScoreShape& shape) {
   auto kernel = &attn_prefill_mfma_kernel<HD, NC, KSPL, BIAS>;
   if (lds > 64 * 1024) {
     static LdsAllowance allowed;
     if (int rc = allow_dynamic_lds(allowed, (const void*)kernel, 150 * 1024); rc != YALM_OK) return rc;
   }
   kernel<<<grid, threads, lds, stream>>>(qp, kp, vp, out, out_f32, lse, cu_seqlens, seq_tile0, tile_order, fold_at, B,
-                                         n_heads, n_kv_heads, window, bias, n_bias);
+                                         n_heads, n_kv_heads, window, shape);
   return launch_status();
 }
 template <int NC, int KSPL, typename... Args>
@@ -344,10 +358,10 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
                                 float* lse,
                                 const int* cu_seqlens, const int* seq_tile0, const int* tile_order, int n_order,
                                 int T, int B, int n_tiles, int n_heads, int n_kv_heads, int head_dim, int window,
-                                const float* bias, int n_bias, hipStream_t stream) {
+                                const ScoreShape& shape, hipStream_t stream) {
   if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || n_tiles > 65535) return YALM_ERR_ARG;
-  if (bias != nullptr && n_bias <= 0) return YALM_ERR_ARG;
-  const bool biased = bias != nullptr;
+  if (shape.bias != nullptr && shape.n_bias <= 0) return YALM_ERR_ARG;
+  const bool biased = shape.any();
   if (tile_order && (n_order <= 0 || n_order > n_tiles)) return YALM_ERR_ARG;
   dim3 grid(n_heads, tile_order ? n_order : n_tiles);
   const long total = (long)grid.x * grid.y;
@@ -365,19 +379,18 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
     // does not matter
     return launch_prefill_hd<1, 2>(head_dim, biased, dim3(n_heads, n_tiles), 512, 4 * tile_bytes, stream, qp, kp, vp,
                                    (bf16*)out, out_f32, lse, cu_seqlens, seq_tile0, (const int*)nullptr, 0, B, n_heads,
-                                   n_kv_heads, window, bias, n_bias);
+                                   n_kv_heads, window, shape);
   }
   if (working <= 2L * compute_units()) {
     // a workgroup of eight waves a compute unit, the workgroups that see the most keys first
     return launch_prefill_hd<2, 2>(head_dim, biased, grid, 512, 4 * tile_bytes, stream, qp, kp, vp, (bf16*)out, out_f32,
                                    lse, cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads, n_kv_heads, window,
-                                   bias, n_bias);
+                                   shape);
   }
   // two workgroups fit a compute unit: with more than one and at most two each, the second
   // half of the launch runs from the shortest workgroup up
   const int cus = compute_units();
   const int fold_at = total > cus && total <= 2 * cus ? cus : (int)total;
   return launch_prefill_hd<2, 1>(head_dim, biased, grid, 256, 2 * tile_bytes, stream, qp, kp, vp, (bf16*)out, out_f32,
-                                 lse, cu_seqlens, seq_tile0, tile_order, fold_at, B, n_heads, n_kv_heads, window, bias,
-                                 n_bias);
+                                 lse, cu_seqlens, seq_tile0, tile_order, fold_at, B, n_heads, n_kv_heads, window, shape);
 }

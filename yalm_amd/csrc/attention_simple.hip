@@ -12,12 +12,12 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
                                 float* lse,
                                 const int* cu_seqlens, const int* seq_tile0, const int* tile_order, int n_order,
                                 int T, int B, int n_tiles, int n_heads, int n_kv_heads, int head_dim, int window,
-                                const float* bias, int n_bias, hipStream_t stream);
+                                const ScoreShape& shape, hipStream_t stream);
 int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                                float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
                                int n_splits, int n_pages, int page_layout, const SinkArgs& sinks,
-                               const int* step_max_len, const int* seq_order, const float* bias, int n_bias,
+                               const int* step_max_len, const int* seq_order, const ScoreShape& shape,
                                hipStream_t stream);
 
 namespace {
@@ -26,8 +26,15 @@ namespace {
 struct ScoreBias {
   const float* table;
   int n;
+  float softcap;               // score <- softcap tanh(score / softcap) before the distance's term (0: no cap)
+  const float* sink_logit;     // [heads]: a logit in the softmax's denominator that has no key and no value (null: none)
   __device__ __forceinline__ float at(int head, int distance) const {
     return table != nullptr ? table[(size_t)head * n + min(max(distance, 0), n - 1)] : 0.f;
+  }
+  // the score of a scaled product at a distance
+  __device__ __forceinline__ float shaped(float s, int head, int distance) const {
+    if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+    return s + at(head, distance);
   }
 };
 
@@ -73,7 +80,7 @@ __global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
       const T* kr = kp + (size_t)lane * hd;
       float d = 0.f;
       for (int i = 0; i < hd; ++i) d = fmaf(qs[i], to_f32(kr[i]), d);
-      s = d / inv + sb.at(h, pos - j);
+      s = sb.shaped(d / inv, h, pos - j);
     }
     float m_new = fmaxf(m, wave_max(s));
     float p = valid ? expf(s - m_new) : 0.f;
@@ -96,6 +103,13 @@ __global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
         acc[a] = acc[a] * corr + s2;
       }
     }
+  }
+  if (sb.sink_logit != nullptr) {                 // the learned logit counts in the denominator only
+    const float sk = sb.sink_logit[h], m_new = fmaxf(m, sk), corr = expf(m - m_new);
+    l = l * corr + expf(sk - m_new);
+    m = m_new;
+#pragma unroll
+    for (int a = 0; a < ACC; ++a) acc[a] *= corr;
   }
 #pragma unroll
   for (int a = 0; a < ACC; ++a) {
@@ -152,7 +166,7 @@ __global__ __launch_bounds__(WAVE) void attn_decode_simple_kernel(
       if (valid) {
         float d = 0.f;
         for (int i = 0; i < hd; ++i) d = fmaf(qs[i], to_f32(kp[page_k_offset(page_layout, lane, i, hd)]), d);
-        s = d / inv + sb.at(h, L - 1 - pos);
+        s = sb.shaped(d / inv, h, L - 1 - pos);
       }
       float m_new = fmaxf(m, wave_max(s));
       float p = valid ? expf(s - m_new) : 0.f;
@@ -197,7 +211,8 @@ template <typename T, bool BASE2 = false, int ACC = ACC_SMALL>
 __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(const float* __restrict__ partial,
                                                                              T* __restrict__ out,
                                                                              float* __restrict__ lse, int n_heads,
-                                                                             int hd, int n_splits, SinkArgs sk) {
+                                                                             int hd, int n_splits, SinkArgs sk,
+                                                                             const float* __restrict__ sink_logit) {
   // One trip to memory: every wave asks for the maxima and denominators of all splits (lanes over
   // splits) and, before it waits for them, for the sums of its own first splits (waves share the
   // splits of the weighted sum and add their parts in a fixed order).
@@ -256,6 +271,9 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(co
   for (int sp = lane + WAVE; sp < n_splits; sp += WAVE) m = fmaxf(m, part[(size_t)sp * stride + hd]);
   m = wave_max(m);
   for (int j = 0; j < n_behind; ++j) m = fmaxf(m, sink_score[j]);
+  // a learned logit in the denominator (no key, no value), in the units of the maxima
+  const float logit = sink_logit != nullptr ? sink_logit[h] * (BASE2 ? 1.4426950408889634f : 1.0f) : -FLT_MAX;
+  if (sink_logit != nullptr) m = fmaxf(m, logit);
   float l = lane < n_splits ? l0 * weight(m0 - m) : 0.f;
   for (int sp = lane + WAVE; sp < n_splits; sp += WAVE) {
     const float* ps = part + (size_t)sp * stride;
@@ -263,6 +281,7 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(co
   }
   l = wave_sum(l);
   for (int j = 0; j < n_behind; ++j) l += weight(sink_score[j] - m);
+  if (sink_logit != nullptr && l > 0.f) l += weight(logit - m);
   const float inv_l = l > 0.f ? 1.0f / l : 0.f;
   if (lse != nullptr && threadIdx.x == 0)
     lse[(size_t)b * n_heads + h] = l > 0.f ? (BASE2 ? m * 0.6931471805599453f : m) + logf(l) : -FLT_MAX;
@@ -314,11 +333,13 @@ extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const v
                                      const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
                                  const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads,
                                  int n_kv_heads, int head_dim, int window, int dtype, int force_simple,
-                                 const float* score_bias, int n_bias, hipStream_t stream) {
+                                 const float* score_bias, int n_bias, float softcap, const float* sink_logit,
+                                 hipStream_t stream) {
   if (T <= 0) return YALM_OK;
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_tiles <= 0) return YALM_ERR_ARG;
-  if (score_bias != nullptr && n_bias <= 0) return YALM_ERR_ARG;
-  const ScoreBias sb = {score_bias, n_bias};
+  if ((score_bias != nullptr && n_bias <= 0) || softcap < 0.f) return YALM_ERR_ARG;
+  const ScoreBias sb = {score_bias, n_bias, softcap, sink_logit};
+  const ScoreShape shape = {score_bias, n_bias, softcap, sink_logit};
   dim3 grid(T, n_heads);
   if (dtype == YALM_F32) {
     if (head_dim <= ACC_SMALL * WAVE)
@@ -334,7 +355,7 @@ extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const v
   if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
   if (!force_simple) {
     int rc = yalm_attn_prefill_bf16_mfma(q, k_stage, v_stage, out, out_f32, lse, cu_seqlens, seq_tile0, tile_order, n_order, T, B,
-                                         n_tiles, n_heads, n_kv_heads, head_dim, window, score_bias, n_bias, stream);
+                                         n_tiles, n_heads, n_kv_heads, head_dim, window, shape, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
   if (head_dim <= ACC_SMALL * WAVE)
@@ -355,19 +376,20 @@ extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void*
                                  hipStream_t stream) {
   return yalm_attn_prefill_lse(q, k_stage, v_stage, out, nullptr, nullptr, cu_seqlens, seq_tile0, tok_seq, tok_pos, tile_order,
                                n_order, T, B, n_tiles, n_heads, n_kv_heads, head_dim, window, dtype, force_simple,
-                               nullptr, 0, stream);
+                               nullptr, 0, 0.f, nullptr, stream);
 }
 
 // merges the partial results of the splits (also used by the MFMA kernel)
 int yalm_attn_decode_combine_bf16(const float* partial, void* out, float* lse, int B, int n_heads, int head_dim,
-                                  int n_splits, int base2, const SinkArgs& sinks, hipStream_t stream) {
+                                  int n_splits, int base2, const SinkArgs& sinks, const float* sink_logit,
+                                  hipStream_t stream) {
   dim3 cgrid(B, n_heads);
   if (base2)
     attn_decode_combine_kernel<bf16, true><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads,
-                                                                                  head_dim, n_splits, sinks);
+                                                                                  head_dim, n_splits, sinks, sink_logit);
   else
     attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads,
-                                                                            head_dim, n_splits, sinks);
+                                                                            head_dim, n_splits, sinks, sink_logit);
   return launch_status();
 }
 
@@ -380,10 +402,13 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
                     int ring_pages, const int* seq_slot, const int* seq_len, void* out, float* lse, float* partial,
                     int B, int n_heads, int n_kv_heads, int head_dim, int window, int n_splits, int n_pages,
                     int page_layout, int dtype, int force_simple, const SinkArgs& sinks, const int* step_max_len,
-                    const int* seq_order, const float* score_bias, int n_bias, hipStream_t stream) {
+                    const int* seq_order, const float* score_bias, int n_bias, float softcap,
+                    const float* sink_logit, hipStream_t stream) {
   if (B <= 0) return YALM_OK;
-  if (score_bias != nullptr && (n_bias <= 0 || sinks.n_sinks > 0)) return YALM_ERR_ARG;   // sinks are scored without it
-  const ScoreBias sb = {score_bias, n_bias};
+  const ScoreShape shape = {score_bias, n_bias, softcap, sink_logit};
+  if ((score_bias != nullptr && n_bias <= 0) || softcap < 0.f || (shape.any() && sinks.n_sinks > 0))
+    return YALM_ERR_ARG;                                                // kept first positions are scored unshaped
+  const ScoreBias sb = {score_bias, n_bias, softcap, sink_logit};
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_splits <= 0 || ring_pages <= 0 ||
       !page_layout_ok(page_layout, head_dim))
     return YALM_ERR_ARG;
@@ -394,13 +419,13 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
           (const float*)q, (const float*)k_pages, (const float*)v_pages, block_table, table_stride, ring_pages,
           seq_slot, seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, sb);
       attn_decode_combine_kernel<float><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (float*)out, lse, n_heads,
-                                                                               head_dim, n_splits, sinks);
+                                                                               head_dim, n_splits, sinks, sink_logit);
     } else {
       attn_decode_simple_kernel<float, ACC_BIG><<<grid, WAVE, 0, stream>>>(
           (const float*)q, (const float*)k_pages, (const float*)v_pages, block_table, table_stride, ring_pages,
           seq_slot, seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, sb);
       attn_decode_combine_kernel<float, false, ACC_BIG><<<cgrid, COMBINE_THREADS, 0, stream>>>(
-          partial, (float*)out, lse, n_heads, head_dim, n_splits, sinks);
+          partial, (float*)out, lse, n_heads, head_dim, n_splits, sinks, sink_logit);
     }
     return launch_status();
   }
@@ -408,7 +433,7 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
   if (!force_simple) {
     int rc = yalm_attn_decode_bf16_mfma(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len,
                                         out, lse, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits,
-                                        n_pages, page_layout, sinks, step_max_len, seq_order, score_bias, n_bias, stream);
+                                        n_pages, page_layout, sinks, step_max_len, seq_order, shape, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
   if (head_dim <= ACC_SMALL * WAVE) {
@@ -416,13 +441,13 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
         (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot,
         seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, sb);
     attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads, head_dim,
-                                                                            n_splits, sinks);
+                                                                            n_splits, sinks, sink_logit);
   } else {
     attn_decode_simple_kernel<bf16, ACC_BIG><<<grid, WAVE, 0, stream>>>(
         (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot,
         seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, sb);
     attn_decode_combine_kernel<bf16, false, ACC_BIG><<<cgrid, COMBINE_THREADS, 0, stream>>>(
-        partial, (bf16*)out, lse, n_heads, head_dim, n_splits, sinks);
+        partial, (bf16*)out, lse, n_heads, head_dim, n_splits, sinks, sink_logit);
   }
   return launch_status();
 }
@@ -433,11 +458,12 @@ extern "C" int yalm_attn_decode_lse(const void* q, const void* k_pages, const vo
                                     void* out, float* lse, float* partial, int B, int n_heads, int n_kv_heads,
                                     int head_dim, int window, int n_splits, int n_pages, int page_layout, int dtype,
                                     int force_simple, const int* step_max_len, const int* seq_order,
-                                    const float* score_bias, int n_bias, hipStream_t stream) {
+                                    const float* score_bias, int n_bias, float softcap, const float* sink_logit,
+                                    hipStream_t stream) {
   SinkArgs none = {};
   return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, lse,
                          partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, dtype,
-                         force_simple, none, step_max_len, seq_order, score_bias, n_bias, stream);
+                         force_simple, none, step_max_len, seq_order, score_bias, n_bias, softcap, sink_logit, stream);
 }
 
 extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -446,7 +472,7 @@ extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* 
                                 int n_splits, int n_pages, int dtype, int force_simple, hipStream_t stream) {
   return yalm_attn_decode_lse(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out,
                               nullptr, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages,
-                              YALM_PAGE_ROWS, dtype, force_simple, nullptr, nullptr, nullptr, 0, stream);
+                              YALM_PAGE_ROWS, dtype, force_simple, nullptr, nullptr, nullptr, 0, 0.f, nullptr, stream);
 }
 
 extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -482,7 +508,7 @@ extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const 
   sk.n_sinks = n_sinks;
   return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, nullptr,
                          partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, dtype,
-                         force_simple, sk, step_max_len, seq_order, nullptr, 0, stream);
+                         force_simple, sk, step_max_len, seq_order, nullptr, 0, 0.f, nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -35,6 +35,48 @@ extern "C" int yalm_embed(const void* table, int table_dtype, const int* tokens,
   return launch_status();
 }
 
+// x[t, :] = table[tokens[t], :] * scale + a sinusoidal position vector: entry 2i is sin(p f_i), entry 2i + 1 the
+// cosine of the same angle.  freq holds the f_i in float64 (made on the host); the angle is formed and brought into
+// one turn in float64, so that it is exact at every position, and sine and cosine are float32's.
+template <typename T>
+__global__ void embed_sinusoid_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
+                                      const int* __restrict__ positions, const double* __restrict__ freq, float scale,
+                                      float* __restrict__ out, int D, int V) {
+  int t = blockIdx.x;
+  int tok = tokens[t];
+  float* o = out + (size_t)t * D;
+  if (tok < 0 || tok >= V) {
+    for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = 0.f;
+    return;
+  }
+  const T* row = table + (size_t)tok * D;
+  const double p = (double)positions[t];
+  for (int i = threadIdx.x; i < D; i += blockDim.x) {
+    float v = to_f32(row[i]) * scale;
+    if (freq != nullptr) {
+      double a = p * freq[i >> 1];
+      a -= floor(a * 0.15915494309189535) * 6.283185307179586;
+      v += (i & 1) ? cosf((float)a) : sinf((float)a);
+    }
+    o[i] = v;
+  }
+}
+
+extern "C" int yalm_embed_sinusoid(const void* table, int table_dtype, const int* tokens, const int* positions,
+                                   const double* freq, float scale, float* out, int T, int D, int V,
+                                   hipStream_t stream) {
+  if (T <= 0) return YALM_OK;
+  if (D <= 0 || V <= 0 || (freq != nullptr && positions == nullptr)) return YALM_ERR_ARG;
+  int threads = D >= 1024 ? 1024 : (D >= 256 ? 256 : 64);
+  if (table_dtype == YALM_F32)
+    embed_sinusoid_kernel<float><<<T, threads, 0, stream>>>((const float*)table, tokens, positions, freq, scale, out, D, V);
+  else if (table_dtype == YALM_BF16)
+    embed_sinusoid_kernel<bf16><<<T, threads, 0, stream>>>((const bf16*)table, tokens, positions, freq, scale, out, D, V);
+  else
+    return YALM_ERR_DTYPE;
+  return launch_status();
+}
+
 // ---------------------------------------------------------------------------
 // RMSNorm: one block per row, sum of squares in float32
 // ---------------------------------------------------------------------------

@@ -46,19 +46,50 @@ __device__ __forceinline__ float dot_row<bf16>(const bf16* __restrict__ w, const
 // logits given (w null, h = float32 logits [T, E]) or made here, a dot product a wave at a time
 template <typename T>
 __global__ __launch_bounds__(WAVE) void moe_route_kernel(const T* __restrict__ h, const T* __restrict__ w, int* __restrict__ ids,
-                                                         float* __restrict__ wts, int D, int E, int top, int renorm) {
+                                                         float* __restrict__ wts, int D, int E, int top, int renorm,
+                                                         const float* __restrict__ bias) {
   __shared__ float score[MOE_MAX_EXPERTS];
   const int t = blockIdx.x, lane = threadIdx.x;
   if (w == nullptr) {
-    for (int e = lane; e < E; e += WAVE) score[e] = to_f32(h[(size_t)t * E + e]);
+    for (int e = lane; e < E; e += WAVE) score[e] = to_f32(h[(size_t)t * E + e]) + (bias != nullptr ? bias[e] : 0.f);
   } else {
     const T* x = h + (size_t)t * D;
     for (int e = 0; e < E; ++e) {
       const float z = wave_sum(dot_row<T>(w + (size_t)e * D, x, D, lane));
-      if (lane == 0) score[e] = z;
+      if (lane == 0) score[e] = z + (bias != nullptr ? bias[e] : 0.f);
     }
   }
   __syncthreads();
+  if (renorm == 2) {
+    // The experts with the largest LOGITS, weighted by the softmax over the chosen logits alone (no score is formed
+    // over all experts, so that a logit far below the largest still takes its place in the order).
+    float first = 0.f, total = 0.f;
+    for (int k = 0; k < top; ++k) {
+      float best = -3.4e38f;
+      int at = 0x7fffffff;
+      for (int e = lane; e < E; e += WAVE) {
+        const float v = score[e];
+        if (v > best) { best = v; at = e; }
+      }
+      for (int o = WAVE / 2; o > 0; o >>= 1) {
+        const float ob = __shfl_xor(best, o, WAVE);
+        const int oa = __shfl_xor(at, o, WAVE);
+        if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+      }
+      if (at == 0x7fffffff) at = 0;               // nothing finite is left
+      if (k == 0) first = best;
+      const float wk = expf(best - first);
+      if (lane == 0) {
+        ids[(size_t)t * top + k] = at;
+        wts[(size_t)t * top + k] = wk;
+        score[at] = -3.4e38f;                     // taken
+      }
+      total += wk;
+      __syncthreads();
+    }
+    for (int k = lane; k < top; k += WAVE) wts[(size_t)t * top + k] /= total;
+    return;
+  }
   float m = -3.0e38f;
   for (int e = lane; e < E; e += WAVE) m = fmaxf(m, score[e]);
   m = wave_max(m);
@@ -96,7 +127,7 @@ __global__ __launch_bounds__(WAVE) void moe_route_kernel(const T* __restrict__ h
 template <typename T>
 __global__ __launch_bounds__(PAIR_WAVES * WAVE) void moe_pair_gate_up_kernel(const T* __restrict__ h, const T* __restrict__ w_gate,
                                                                              const T* __restrict__ w_up, const int* __restrict__ ids,
-                                                                             float limit, float alpha, T* __restrict__ mid, int top,
+                                                                             float limit, float alpha, float up_shift, T* __restrict__ mid, int top,
                                                                              int D, int F, int E) {
   const int pair = blockIdx.x;
   const int e = ids[pair];
@@ -112,7 +143,7 @@ __global__ __launch_bounds__(PAIR_WAVES * WAVE) void moe_pair_gate_up_kernel(con
       g = fminf(g, limit);
       u = fminf(fmaxf(u, -limit), limit);
     }
-    if (lane == 0) mid[(size_t)pair * F + f] = from_f32<T>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+    if (lane == 0) mid[(size_t)pair * F + f] = from_f32<T>(g / (1.0f + expf(-alpha * g)) * (u + up_shift));
   }
 }
 
@@ -210,7 +241,7 @@ template <bool GATED>
 __global__ __launch_bounds__(GR_THREADS, 2) void moe_grouped_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W0,
                                                                     const bf16* __restrict__ W1, const int* __restrict__ tile_expert,
                                                                     const int* __restrict__ pair_of_row, int top, void* __restrict__ Cv,
-                                                                    int N, int K, float limit, float alpha) {
+                                                                    int N, int K, float limit, float alpha, float up_shift) {
   const int e = tile_expert[blockIdx.y];
   if (e < 0) return;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -313,7 +344,7 @@ __global__ __launch_bounds__(GR_THREADS, 2) void moe_grouped_kernel(const bf16* 
             g = fminf(g, limit);
             u = fminf(fmaxf(u, -limit), limit);
           }
-          ((bf16*)Cv)[(size_t)row * N + f] = static_cast<bf16>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+          ((bf16*)Cv)[(size_t)row * N + f] = static_cast<bf16>(g / (1.0f + expf(-alpha * g)) * (u + up_shift));
         }
       } else {
 #pragma unroll
@@ -348,34 +379,35 @@ extern "C" int yalm_moe_route(const void* h, const void* w_router, int dtype, in
   if (T <= 0) return YALM_OK;
   if (D <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > E) return YALM_ERR_ARG;
   if (dtype == YALM_BF16)
-    moe_route_kernel<bf16><<<T, WAVE, 0, stream>>>((const bf16*)h, (const bf16*)w_router, ids, wts, D, E, top, renorm);
+    moe_route_kernel<bf16><<<T, WAVE, 0, stream>>>((const bf16*)h, (const bf16*)w_router, ids, wts, D, E, top, renorm, nullptr);
   else if (dtype == YALM_F32)
-    moe_route_kernel<float><<<T, WAVE, 0, stream>>>((const float*)h, (const float*)w_router, ids, wts, D, E, top, renorm);
+    moe_route_kernel<float><<<T, WAVE, 0, stream>>>((const float*)h, (const float*)w_router, ids, wts, D, E, top, renorm, nullptr);
   else
     return YALM_ERR_DTYPE;
   return launch_status();
 }
 
-extern "C" int yalm_moe_select(const float* logits, int* ids, float* wts, int T, int E, int top, int renorm,
-                               hipStream_t stream) {
+extern "C" int yalm_moe_select(const float* logits, const float* bias, int* ids, float* wts, int T, int E, int top,
+                               int renorm, hipStream_t stream) {
   if (T <= 0) return YALM_OK;
   if (E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > E) return YALM_ERR_ARG;
-  moe_route_kernel<float><<<T, WAVE, 0, stream>>>(logits, nullptr, ids, wts, E, E, top, renorm);
+  if (renorm < 0 || renorm > 2) return YALM_ERR_ARG;
+  moe_route_kernel<float><<<T, WAVE, 0, stream>>>(logits, nullptr, ids, wts, E, E, top, renorm, bias);
   return launch_status();
 }
 
 extern "C" int yalm_moe_pair_gate_up(const void* h, const void* w_gate, const void* w_up, const int* ids, float limit,
-                                     float alpha, void* mid, int T, int top, int D, int F, int E, int dtype,
+                                     float alpha, float up_shift, void* mid, int T, int top, int D, int F, int E, int dtype,
                                      hipStream_t stream) {
   if (T <= 0) return YALM_OK;
   if (D <= 0 || F <= 0 || E <= 0 || top <= 0) return YALM_ERR_ARG;
   dim3 grid(T * top, ceil_div(F, PAIR_ROWS));
   if (dtype == YALM_BF16)
     moe_pair_gate_up_kernel<bf16><<<grid, PAIR_WAVES * WAVE, 0, stream>>>((const bf16*)h, (const bf16*)w_gate, (const bf16*)w_up,
-                                                                          ids, limit, alpha, (bf16*)mid, top, D, F, E);
+                                                                          ids, limit, alpha, up_shift, (bf16*)mid, top, D, F, E);
   else if (dtype == YALM_F32)
     moe_pair_gate_up_kernel<float><<<grid, PAIR_WAVES * WAVE, 0, stream>>>((const float*)h, (const float*)w_gate,
-                                                                           (const float*)w_up, ids, limit, alpha, (float*)mid,
+                                                                           (const float*)w_up, ids, limit, alpha, up_shift, (float*)mid,
                                                                            top, D, F, E);
   else
     return YALM_ERR_DTYPE;
@@ -404,7 +436,7 @@ extern "C" int yalm_moe_pair_down(const void* mid, const void* w_down, const int
 extern "C" int yalm_moe_grouped_tiles(int n_pairs, int E) { return ceil_div(n_pairs, GR_TM) + E; }
 
 extern "C" int yalm_moe_grouped(const void* h, const void* w_gate, const void* w_up, const void* w_down, const int* ids,
-                                const float* wts, float limit, float alpha, int* pair_of_row, int* row_of_pair,
+                                const float* wts, float limit, float alpha, float up_shift, int* pair_of_row, int* row_of_pair,
                                 int* tile_expert, void* mid, float* y, float* out, int T, int top, int D, int F, int E,
                                 int accumulate, hipStream_t stream) {
   if (T <= 0) return YALM_OK;
@@ -418,9 +450,9 @@ extern "C" int yalm_moe_grouped(const void* h, const void* w_gate, const void* w
   moe_group_kernel<<<1, GROUP_THREADS, 0, stream>>>(ids, (int)n_pairs, E, max_tiles, pair_of_row, row_of_pair, tile_expert);
   const size_t lds = (size_t)(GR_TM + GR_TN) * GR_ROW * sizeof(bf16);
   moe_grouped_kernel<true><<<dim3(ceil_div(F, GR_TN / 2), max_tiles), GR_THREADS, lds, stream>>>(
-      (const bf16*)h, (const bf16*)w_gate, (const bf16*)w_up, tile_expert, pair_of_row, top, mid, F, D, limit, alpha);
+      (const bf16*)h, (const bf16*)w_gate, (const bf16*)w_up, tile_expert, pair_of_row, top, mid, F, D, limit, alpha, up_shift);
   moe_grouped_kernel<false><<<dim3(ceil_div(D, GR_TN), max_tiles), GR_THREADS, lds, stream>>>(
-      (const bf16*)mid, (const bf16*)w_down, nullptr, tile_expert, pair_of_row, top, y, D, F, 0.f, 0.f);
+      (const bf16*)mid, (const bf16*)w_down, nullptr, tile_expert, pair_of_row, top, y, D, F, 0.f, 0.f, 0.f);
   moe_combine_kernel<<<T, 256, 0, stream>>>(y, row_of_pair, wts, out, top, D, accumulate);
   return launch_status();
 }

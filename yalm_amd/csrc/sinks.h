@@ -6,6 +6,23 @@
 
 #define YALM_MAX_SINKS 16
 
+// What shapes a score between the product q . k / sqrt(head size) and the softmax, beside the mask: a cap
+// (score <- cap tanh(score / cap); 0: none), then a term by the distance of query and key, bias[head][min(distance,
+// n_bias - 1)] (null: none), and a learned logit per head that stands in the softmax's denominator without a key or a
+// value of its own (sink_logit[head], null: none; it is neither scaled nor capped and gets no distance term).
+struct ScoreShape {
+  const float* bias;
+  int n_bias;
+  float softcap;
+  const float* sink_logit;
+  __host__ __device__ bool any() const { return bias != nullptr || softcap > 0.f || sink_logit != nullptr; }
+};
+// cap tanh(s / cap) from the exponential instruction (the matrix-core kernels; absolute error about 1e-7 cap)
+__device__ __forceinline__ float soft_cap_fast(float s, float cap) {
+  const float e = __builtin_amdgcn_exp2f(s * (2.0f * 1.4426950408889634f / cap));
+  return cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e));
+}
+
 // What a decode step's merge of the attention splits needs to take the sinks in (n_sinks 0: none).
 struct SinkArgs {
   const void* q;              // [B, n_heads, hd], rotated at each token's position

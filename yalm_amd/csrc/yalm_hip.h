@@ -165,17 +165,20 @@ long yalm_attn_decode_workspace(int B, int n_heads, int head_dim, int n_splits);
 // score_bias (device, float32 [n_heads, n_bias]; may be null): a term added to every score (after the 1/sqrt(head_dim)
 // scaling) by the distance between query and key, score_bias[head, min(distance, n_bias - 1)]: what a position
 // encoding that is no rotation needs (not together with attention sinks).
+// softcap (0: none): score <- softcap tanh(score / softcap), after the scaling and before score_bias's term.
+// sink_logit (device, float32 [n_heads]; may be null): a learned logit per head that counts once in the softmax's
+// denominator and has no key and no value (it is not scaled, not capped and gets no distance term; lse counts it).
 int yalm_attn_prefill_lse(const void* q, const void* k_stage, const void* v_stage, void* out, float* out_f32, float* lse,
                           const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
                           const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads, int n_kv_heads,
                           int head_dim, int window, int dtype, int force_simple, const float* score_bias, int n_bias,
-                          hipStream_t stream);
+                          float softcap, const float* sink_logit, hipStream_t stream);
 int yalm_attn_decode_lse(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                          int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                          float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
                          int n_splits, int n_pages, int page_layout, int dtype, int force_simple,
                          const int* step_max_len, const int* seq_order, const float* score_bias, int n_bias,
-                         hipStream_t stream);
+                         float softcap, const float* sink_logit, hipStream_t stream);
 
 // Attention sinks beside a window (src/infer.cpp:305-319, 486-488): the first n_sinks positions of a
 // sequence stay visible when the window has moved past them, and each then counts as lying
@@ -279,9 +282,14 @@ int yalm_latent_pack(const float* proj, long proj_row, int q_head, int q_rot_off
 int yalm_moe_route(const void* h, const void* w_router, int dtype, int* ids, float* wts, int T, int D, int E, int top,
                    int renorm, hipStream_t stream);
 // The same choice from logits that a product has made already (float32 [T, E]).
-int yalm_moe_select(const float* logits, int* ids, float* wts, int T, int E, int top, int renorm, hipStream_t stream);
+// bias (float32 [E], may be null) is added to the logits first.  renorm 2: the experts with the largest logits,
+// weighted by the softmax over the chosen logits alone.
+int yalm_moe_select(const float* logits, const float* bias, int* ids, float* wts, int T, int E, int top, int renorm,
+                    hipStream_t stream);
+// up_shift: the number added to the clamped up value (mid = g sigmoid(alpha g) (u + up_shift); the text above has 1;
+// alpha 1, limit 0 and up_shift 0 give silu(gate) * up).
 int yalm_moe_pair_gate_up(const void* h, const void* w_gate, const void* w_up, const int* ids, float limit, float alpha,
-                          void* mid, int T, int top, int D, int F, int E, int dtype, hipStream_t stream);
+                          float up_shift, void* mid, int T, int top, int D, int F, int E, int dtype, hipStream_t stream);
 int yalm_moe_pair_down(const void* mid, const void* w_down, const int* ids, const float* wts, float* out, int T, int top,
                        int D, int F, int E, int dtype, int accumulate, hipStream_t stream);
 
@@ -291,9 +299,36 @@ int yalm_moe_pair_down(const void* mid, const void* w_down, const int* ids, cons
 // tile_expert int32 [max_tiles], mid bfloat16 [max_tiles * 128, F], y float32 [max_tiles * 128, D].
 int yalm_moe_grouped_tiles(int n_pairs, int E);
 int yalm_moe_grouped(const void* h, const void* w_gate, const void* w_up, const void* w_down, const int* ids,
-                     const float* wts, float limit, float alpha, int* pair_of_row, int* row_of_pair, int* tile_expert,
-                     void* mid, float* y, float* out, int T, int top, int D, int F, int E, int accumulate,
+                     const float* wts, float limit, float alpha, float up_shift, int* pair_of_row, int* row_of_pair,
+                     int* tile_expert, void* mid, float* y, float* out, int T, int top, int D, int F, int E, int accumulate,
                      hipStream_t stream);
+
+// x[t, :] = table[tokens[t], :] * scale + (freq not null) a sinusoidal position vector: entry 2i is sin(p f_i), entry
+// 2i + 1 cos(p f_i), p = positions[t], f = freq (float64 [ceil(D / 2)] on the device).  A negative token gives zeros.
+int yalm_embed_sinusoid(const void* table, int table_dtype, const int* tokens, const int* positions, const double* freq,
+                        float scale, float* out, int T, int D, int V, hipStream_t stream);
+
+// Between the q/k/v product and an attention without rotation (qkv_pack.hip): qkv float32 [T, H d + G d + G dv]
+// (+ bias, float32 of that width or null); RMS norms over the whole query and key projections with the weights w_q
+// [H d], w_k [G d] (float32; null: no norm); the queries times q_scale and, with temp_every > 0, times 1 + temp_coef
+// ln(floor((p + 1) / temp_every) + 1); blend 1 stores the values in v_first (float32 [T, G dv]), blend 2 replaces them
+// by (1 - lam) v + lam v_first (lam: one float32 on the device).  Heads are written `pad` wide with zeros behind
+// (pad >= d, dv): q_out [T, H, pad]; keys and values into the cache pages (page_layout of head size pad) and, with
+// k_stage, into the staging tiles of a step of whole prompts, as yalm_rope_kv_write does.
+int yalm_qkv_pack(const float* qkv, const float* bias, const float* w_q, const float* w_k, float eps, float temp_coef,
+                  int temp_every, float q_scale, float* v_first, int blend, const float* lam, void* q_out, void* k_stage,
+                  void* v_stage, const int* seq_tile0, void* k_pages, void* v_pages, const int* block_table,
+                  int table_stride, int ring_pages, const int* tok_seq, const int* tok_pos, const int* seq_slot,
+                  const int* seq_len, int T, int n_heads, int n_kv_heads, int d, int dv, int pad, int n_pages,
+                  int page_layout, int dtype, hipStream_t stream);
+
+// The matrix-memory recurrence (mlstm.hip): proj float32 [T, 2 H d + 2 H dv + 2 H] = q | k | v | g | z_i | z_f of
+// every token; state float32 [n_slots, H, d dv + d + 1] (S, n, m of every head), read and left advanced; out `dtype`
+// [T, H dv] = the heads' results divided by their root mean square, times w_norm, times sigmoid(g).  The tokens of
+// sequence b are rows cu_seqlens[b] .. cu_seqlens[b + 1] - 1; seq_slot[b] < 0: a padding row, left alone.
+int yalm_mlstm_scan(const float* proj, const float* b_i, const float* b_f, const float* w_norm, float* state,
+                    const int* cu_seqlens, const int* seq_slot, void* out, int B, int H, int d, int dv, float q_scale,
+                    float cap, float floor_, float eps, int n_slots, int dtype, hipStream_t stream);
 
 // Yardsticks for the measurement (probes.hip): a kernel that only reads `bytes` bytes once with `workgroups`
 // workgroups (out: 1,024 words of scratch), and a loop of matrix-core instructions on registers (shape 32:

@@ -86,6 +86,19 @@ def embed(table, tokens, out):
     return out
 
 
+def embed_sinusoid(table, tokens, positions, freq, scale, out):
+    """out[t] = float(table[tokens[t]]) * scale + (freq given) the sinusoidal vector of positions[t]: entry 2i is
+    sin(p freq[i]), entry 2i + 1 the cosine; freq float64 [ceil(D / 2)] on the device.  A negative token gives zeros."""
+    V, D = table.shape
+    T = tokens.shape[0]
+    p_freq = None if freq is None else _need(freq, "freq", torch.float64, ((D + 1) // 2,))
+    p_pos = None if freq is None else _need(positions, "positions", torch.int32, (T,))
+    library.check(library.lib().yalm_embed_sinusoid(
+        _need(table, "table"), dtype_code(table.dtype), _need(tokens, "tokens", torch.int32, (T,)), p_pos, p_freq,
+        float(scale), _need(out, "out", torch.float32, (T, D)), T, D, V, _stream()), "embed_sinusoid")
+    return out
+
+
 def rmsnorm(x, weight, out, eps, row_index=None):
     """out[r] = x[row_index[r] or r] * rsqrt(mean(x^2) + eps) * weight."""
     D = x.shape[-1]
@@ -567,13 +580,24 @@ def _bias(score_bias, n_heads):
     return _need(score_bias, "score_bias", torch.float32, (n_heads, n)), n
 
 
+def _shape(softcap, sink_logit, n_heads):
+    """(cap, address of the sink logits): softcap > 0 replaces every scaled score s by softcap tanh(s / softcap) before
+    the score bias; sink_logit, float32 [n_heads] on the device, is a logit per head that counts once in the softmax's
+    denominator and has neither key nor value."""
+    cap = float(softcap or 0.0)
+    if cap < 0.0:
+        raise ValueError("a score cap must be positive (0: none)")
+    return cap, _opt(sink_logit, "sink_logit", torch.float32, (n_heads,))
+
+
 def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_pos, n_heads, n_kv_heads, head_dim,
-                 window, tile_order=None, lse=None, out_f32=None, score_bias=None):
+                 window, tile_order=None, lse=None, out_f32=None, score_bias=None, softcap=0.0, sink_logit=None):
     """Causal (and windowed) attention of packed sequences that start at position 0, over
     the keys and values that rope_kv_write staged for this step.  tile_order (device int32,
     from prefill_tile_order) only changes the order of the work.  lse (float32 [T, n_heads], optional)
     receives the logarithm of every query's sum of exp(score), for attn_sink_mix; out_f32 (float32 [T, n_heads *
-    head_dim], optional) the result before it is rounded to out's dtype, for the same.  score_bias: see _bias."""
+    head_dim], optional) the result before it is rounded to out's dtype, for the same.  score_bias: see _bias;
+    softcap, sink_logit: see _shape."""
     _check_heads(n_heads, n_kv_heads, head_dim)
     T = q.shape[0]
     dt = q.dtype
@@ -596,7 +620,8 @@ def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_p
     library.check(library.lib().yalm_attn_prefill_lse(p_q, p_k, p_v, p_o, p_o32, p_lse, p_cu, p_t0, p_ts, p_tp, p_or, n_order,
                                                       T, B, n_tiles, n_heads, n_kv_heads, head_dim, int(window),
                                                       dtype_code(dt), 1 if FORCE_SIMPLE else 0,
-                                                      *_bias(score_bias, n_heads), _stream()),
+                                                      *_bias(score_bias, n_heads), *_shape(softcap, sink_logit, n_heads),
+                                                      _stream()),
                   "attn_prefill")
     return out
 
@@ -607,13 +632,13 @@ def attn_decode_workspace_floats(B, n_heads, head_dim, n_splits):
 
 def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len, out, partial, n_heads, n_kv_heads,
                 head_dim, window, n_splits, lse=None, sinks=None, layout=None, step_max_len=None, seq_order=None,
-                score_bias=None):
+                score_bias=None, softcap=0.0, sink_logit=None):
     """One query per sequence over the cache pages (laid out as `layout` says, default page_layout(head_dim));
     seq_len counts the new key.  lse as in attn_prefill.  step_max_len (int32 [1] on the device, optional): the
     length of the step's longest sequence, with which sequences of unequal lengths are cut into splits of equal
     size; seq_order (int32 [B] on the device, a permutation of the rows, optional): the order in which the
-    workgroups take the rows (both change the division of the work and no result).  score_bias: see _bias (not with
-    sinks).
+    workgroups take the rows (both change the division of the work and no result).  score_bias: see _bias; softcap,
+    sink_logit: see _shape (none of the three with sinks).
     sinks = (sink_k, sink_v [slots, n_kv_heads, n_sinks, head_dim], cos_sin or None, rotary_dim, store):
     the attention sinks that a query's window no longer covers are taken in where the splits are merged
     (their keys turned by max(0, position - window - n_sinks + 1) positions with the table cos_sin); with
@@ -644,12 +669,12 @@ def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len,
         library.check(library.lib().yalm_attn_decode_lse(
             p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_ss, p_sl, p_o, p_lse, p_w, B, n_heads, n_kv_heads, head_dim,
             int(window), int(n_splits), n_pages, _layout(layout, head_dim), dtype_code(dt), force, p_max, p_ord,
-            *_bias(score_bias, n_heads), _stream()), "attn_decode")
+            *_bias(score_bias, n_heads), *_shape(softcap, sink_logit, n_heads), _stream()), "attn_decode")
         return out
     if lse is not None:
         raise ValueError("attn_decode leaves no lse when it takes the sinks in itself")
-    if score_bias is not None:
-        raise ValueError("attention sinks are scored without a score bias: the two do not go together")
+    if score_bias is not None or softcap or sink_logit is not None:
+        raise ValueError("attention sinks are scored without a score bias, a cap or a sink logit: they do not go together")
     sink_k, sink_v, cos_sin, rotary_dim, store = sinks
     n_slots, _, n_sinks, _ = sink_k.shape
     if window < n_sinks:
@@ -821,6 +846,79 @@ def latent_pack(proj, q_head, q_rot_off, kv_off, norm_w, eps, q_scale, out, n_he
     return out
 
 
+def qkv_pack(qkv, bias, w_q, w_k, eps, q_temp, q_scale, v_first, blend, lam, q_out, k_stage, v_stage, seq_tile0, k_pages,
+             v_pages, block_table, ring_pages, tok_seq, tok_pos, seq_slot, seq_len, n_heads, n_kv_heads, d, dv, pad):
+    """From a q/k/v product to an attention without rotation.  qkv float32 [T, H d + G d + G dv] (+ bias, float32 of
+    that width or None); RMS norms over the WHOLE query and key projections with the weights w_q [H d], w_k [G d]
+    (float32; None: no norm); the queries times q_scale and, with q_temp = (coef, every), times 1 + coef ln(floor((p + 1)
+    / every) + 1) at position p; blend 1 stores the values in v_first (float32 [T, G dv]), blend 2 replaces them by
+    (1 - lam) v + lam v_first (lam: one float32 on the device).  Heads are written `pad` wide, zeros behind: q_out [T,
+    H pad]; keys and values into the cache pages (None: nowhere) and, with k_stage, into the staging tiles of a step of
+    whole prompts."""
+    T = qkv.shape[0]
+    Q, K, V = n_heads * d, n_kv_heads * d, n_kv_heads * dv
+    N = Q + K + V
+    dt = q_out.dtype
+    if pad < max(d, dv) or N * 4 > 64 * 1024:
+        raise ValueError("qkv_pack: heads of %d and %d do not fit %d, or a row of %d values is too wide" % (d, dv, pad, N))
+    if blend not in (0, 1, 2) or (blend and v_first is None) or (blend == 2 and lam is None):
+        raise ValueError("qkv_pack: blend %r needs v_first (and lam)" % (blend,))
+    coef, every = q_temp if q_temp else (0.0, 0)
+    n_pages = 0 if k_pages is None else k_pages.shape[0]
+    n_tiles = 0 if k_stage is None else k_stage.shape[0]
+    stride = 0
+    if k_pages is not None:
+        stride = block_table.shape[1]
+        if ring_pages <= 0 or ring_pages > stride:
+            raise ValueError("ring_pages %d does not fit the block table (%d columns)" % (ring_pages, stride))
+    library.check(library.lib().yalm_qkv_pack(
+        _need(qkv, "qkv", torch.float32, (T, N)), _opt(bias, "bias", torch.float32, (N,)),
+        _opt(w_q, "w_q", torch.float32, (Q,)), _opt(w_k, "w_k", torch.float32, (K,)), float(eps), float(coef), int(every),
+        float(q_scale), _opt(v_first, "v_first", torch.float32, (T, V)), int(blend), _opt(lam, "lam", torch.float32),
+        _need(q_out, "q_out", dt, (T, n_heads * pad)),
+        _opt(k_stage, "k_stage", dt, (n_tiles, n_kv_heads, PAGE, pad)),
+        _opt(v_stage, "v_stage", dt, (n_tiles, n_kv_heads, pad, PAGE)),
+        _opt(seq_tile0, "seq_tile0", torch.int32), _opt(k_pages, "k_pages", dt, (n_pages, n_kv_heads, PAGE, pad)),
+        _opt(v_pages, "v_pages", dt, (n_pages, n_kv_heads, pad, PAGE)), _opt(block_table, "block_table", torch.int32, (None, None)),
+        stride, int(ring_pages), _need(tok_seq, "tok_seq", torch.int32, (T,)), _need(tok_pos, "tok_pos", torch.int32, (T,)),
+        _need(seq_slot, "seq_slot", torch.int32), _opt(seq_len, "seq_len", torch.int32), T, n_heads, n_kv_heads, d, dv, pad,
+        n_pages, page_layout(pad), dtype_code(dt), _stream()), "qkv_pack")
+    return q_out
+
+
+MLSTM_MAX_VDIM = 256             # a thread of the recurrence's workgroup owns one column of the state
+MLSTM_MAX_LDS = 150 * 1024
+
+
+def mlstm_fits(d, dv):
+    """Whether mlstm_scan takes heads of these sizes (the state of a head waits in LDS)."""
+    groups = max(1, min(256 // max(dv, 1), d))
+    return 0 < dv <= MLSTM_MAX_VDIM and d > 0 and (d * dv + 3 * d + dv + groups * dv) * 4 <= MLSTM_MAX_LDS
+
+
+def mlstm_scan(proj, b_i, b_f, w_norm, state, cu_seqlens, seq_slot, out, n_heads, d, dv, q_scale, cap, floor, eps):
+    """The matrix-memory recurrence over the tokens of a step.  proj float32 [T, 2 H d + 2 H dv + 2 H] = q | k | v | g |
+    z_i | z_f; with i = cap tanh((z_i + b_i) / cap), f = logsigmoid(cap tanh((z_f + b_f) / cap)) (cap 0: uncapped):
+    m' = max(f + m, i), S' = exp(f + m - m') S + exp(i - m') k v^T, n' likewise with k, o = S'^T (q q_scale) / (max(|n' .
+    q|, exp(-m')) + floor); out [T, H dv] = o / rms(o) (a head at a time) * w_norm * sigmoid(g).  state float32
+    [slots, H (d dv + d + 1)] is read and left advanced; the tokens of sequence b are the rows cu_seqlens[b] ..
+    cu_seqlens[b + 1] - 1, in order; rows with seq_slot < 0 are left alone."""
+    T = proj.shape[0]
+    B = seq_slot.shape[0]
+    H = n_heads
+    if not mlstm_fits(d, dv):
+        raise ValueError("mlstm_scan: heads of %d x %d are not offered" % (d, dv))
+    n_slots = state.shape[0]
+    library.check(library.lib().yalm_mlstm_scan(
+        _need(proj, "proj", torch.float32, (T, 2 * H * d + 2 * H * dv + 2 * H)), _need(b_i, "b_i", torch.float32, (H,)),
+        _need(b_f, "b_f", torch.float32, (H,)), _need(w_norm, "w_norm", torch.float32, (H * dv,)),
+        _need(state, "state", torch.float32, (n_slots, H * (d * dv + d + 1))),
+        _need(cu_seqlens, "cu_seqlens", torch.int32, (B + 1,)), _need(seq_slot, "seq_slot", torch.int32, (B,)),
+        _need(out, "out", None, (T, H * dv)), B, H, d, dv, float(q_scale), float(cap), float(floor), float(eps), n_slots,
+        dtype_code(out.dtype), _stream()), "mlstm_scan")
+    return out
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # mixture of experts
 MOE_MAX_EXPERTS = 1024
@@ -840,28 +938,32 @@ def moe_route(h, w_router, ids, wts, renormalize=False):
         1 if renormalize else 0, _stream()), "moe_route")
 
 
-def moe_select(logits, ids, wts, renormalize=False):
-    """moe_route from logits that a product has made already (float32 [T, E])."""
+def moe_select(logits, ids, wts, renormalize=False, bias=None):
+    """moe_route from logits that a product has made already (float32 [T, E]); bias (float32 [E]) is added to them
+    first.  renormalize "chosen": the experts with the largest logits, weighted by the softmax over the chosen logits
+    alone (no score over all experts is formed)."""
     T, E = logits.shape
     top = ids.shape[1]
     if not 0 < top <= E or E > MOE_MAX_EXPERTS:
         raise ValueError("moe_select: %d of %d experts is not offered (at most %d experts)" % (top, E, MOE_MAX_EXPERTS))
+    mode = 2 if renormalize == "chosen" else (1 if renormalize else 0)
     library.check(library.lib().yalm_moe_select(
-        _need(logits, "logits", torch.float32, (T, E)), _need(ids, "ids", torch.int32, (T, top)),
-        _need(wts, "wts", torch.float32, (T, top)), T, E, top, 1 if renormalize else 0, _stream()), "moe_select")
+        _need(logits, "logits", torch.float32, (T, E)), _opt(bias, "bias", torch.float32, (E,)),
+        _need(ids, "ids", torch.int32, (T, top)), _need(wts, "wts", torch.float32, (T, top)), T, E, top, mode, _stream()),
+        "moe_select")
 
 
-def moe_pair_gate_up(h, w_gate, w_up, ids, limit, alpha, mid):
-    """mid[t * top + k] = g sigmoid(alpha g) (u + 1), g = min(w_gate[e] h[t], limit), u = clamp(w_up[e] h[t], +-limit)
-    for e = ids[t, k] (limit <= 0: unclamped); w_gate, w_up [E, F, D]."""
+def moe_pair_gate_up(h, w_gate, w_up, ids, limit, alpha, mid, up_shift=1.0):
+    """mid[t * top + k] = g sigmoid(alpha g) (u + up_shift), g = min(w_gate[e] h[t], limit), u = clamp(w_up[e] h[t], +-limit)
+    for e = ids[t, k] (limit <= 0: unclamped; alpha 1, up_shift 0: silu(gate) * up); w_gate, w_up [E, F, D]."""
     T, D = h.shape
     E, F, _ = w_gate.shape
     top = ids.shape[1]
     dt = h.dtype
     library.check(library.lib().yalm_moe_pair_gate_up(
         _need(h, "h", dt, (T, D)), _need(w_gate, "w_gate", dt, (E, F, D)), _need(w_up, "w_up", dt, (E, F, D)),
-        _need(ids, "ids", torch.int32, (T, top)), float(limit), float(alpha), _need(mid, "mid", dt, (T * top, F)),
-        T, top, D, F, E, dtype_code(dt), _stream()), "moe_pair_gate_up")
+        _need(ids, "ids", torch.int32, (T, top)), float(limit), float(alpha), float(up_shift),
+        _need(mid, "mid", dt, (T * top, F)), T, top, D, F, E, dtype_code(dt), _stream()), "moe_pair_gate_up")
     return mid
 
 
@@ -892,7 +994,7 @@ def moe_grouped_tiles(n_pairs, n_experts):
     return library.lib().yalm_moe_grouped_tiles(int(n_pairs), int(n_experts))
 
 
-def moe_grouped(h, w_gate, w_up, w_down, ids, wts, limit, alpha, scratch, out, accumulate=False):
+def moe_grouped(h, w_gate, w_up, w_down, ids, wts, limit, alpha, scratch, out, accumulate=False, up_shift=1.0):
     """What moe_pair_gate_up + moe_pair_down compute, for many tokens (bfloat16): the pairs are grouped by expert on
     the device and every product is one launch over all experts' tiles on the matrix cores.  scratch(name, shape,
     dtype) hands out the buffers (pair_of_row, row_of_pair, tile_expert, mid, y)."""
@@ -910,7 +1012,7 @@ def moe_grouped(h, w_gate, w_up, w_down, ids, wts, limit, alpha, scratch, out, a
     library.check(library.lib().yalm_moe_grouped(
         _need(h, "h", dt, (T, D)), _need(w_gate, "w_gate", dt, (E, F, D)), _need(w_up, "w_up", dt, (E, F, D)),
         _need(w_down, "w_down", dt, (E, D, F)), _need(ids, "ids", torch.int32, (T, top)),
-        _need(wts, "wts", torch.float32, (T, top)), float(limit), float(alpha),
+        _need(wts, "wts", torch.float32, (T, top)), float(limit), float(alpha), float(up_shift),
         _need(pair_of_row, "pair_of_row", torch.int32, (rows,)), _need(row_of_pair, "row_of_pair", torch.int32, (T * top,)),
         _need(tile_expert, "tile_expert", torch.int32, (tiles,)), _need(mid, "mid", dt, (rows, F)),
         _need(y, "y", torch.float32, (rows, D)), _need(out, "out", torch.float32, (T, D)), T, top, D, F, E,

@@ -34,9 +34,9 @@ _SIGNATURES = {
     "yalm_attn_decode": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_decode_workspace": (ctypes.c_long, [_I, _I, _I, _I]),
     "yalm_attn_prefill_lse": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I,
-                                   _P, _I, _P]),
+                                   _P, _I, _F, _P, _P]),
     "yalm_attn_decode_lse": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P,
-                                  _P, _I, _P]),
+                                  _P, _I, _F, _P, _P]),
     "yalm_sink_store": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_sink_mix": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_decode_sinks": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P]),
@@ -57,16 +57,20 @@ _SIGNATURES = {
                                    _I, _I, _I, _I, _P]),
     "yalm_latent_pack": (_I, [_P, ctypes.c_long, _I, _I, _I, _P, _I, _F, _F, _P, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_moe_route": (_I, [_P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _P]),
-    "yalm_moe_select": (_I, [_P, _P, _P, _I, _I, _I, _I, _P]),
-    "yalm_moe_pair_gate_up": (_I, [_P, _P, _P, _P, _F, _F, _P, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_moe_select": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "yalm_moe_pair_gate_up": (_I, [_P, _P, _P, _P, _F, _F, _F, _P, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_moe_pair_down": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_moe_grouped_tiles": (_I, [_I, _I]),
-    "yalm_moe_grouped": (_I, [_P, _P, _P, _P, _P, _P, _F, _F, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_moe_grouped": (_I, [_P, _P, _P, _P, _P, _P, _F, _F, _F, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_embed_sinusoid": (_I, [_P, _I, _P, _P, _P, _F, _P, _I, _I, _I, _P]),
+    "yalm_qkv_pack": (_I, [_P, _P, _P, _P, _F, _F, _I, _F, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P,
+                           _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_mlstm_scan": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _F, _F, _I, _I, _P]),
     "yalm_probe_read": (_I, [_P, ctypes.c_long, _P, _I, _P]),
     "yalm_probe_mfma": (_I, [_I, _I, _I, _P, _P, _P]),
 }
 
-ABI_VERSION = 28
+ABI_VERSION = 29
 
 
 class KernelError(RuntimeError):

@@ -40,6 +40,39 @@ class PreNormResidualBlock(Part):
             self.feed_forward.forward(h, x, ctx)
 
 
+@part("block", "parallel_residual")
+class ParallelResidualBlock(Part):
+    """x += mixer(h) + feed_forward(h) with h = norm(x): one norm, and both sublayers read its output.  Members: norm,
+    mixer, and optionally feed_forward.  Each sublayer adds its result to the float32 stream in the epilogue of its
+    last product, the mixer first."""
+
+    def __init__(self, layer_spec, dim, prefix=""):
+        super().__init__(None, dim, layer_spec.prefix)
+        p = layer_spec.prefix
+        self.norm = build_part("norm", layer_spec.norm, dim, p)
+        self.mixer = build_part("mixer", layer_spec.mixer, dim, p)
+        self.feed_forward = None
+        if layer_spec.part("feed_forward") is not None:
+            self.feed_forward = build_part("feed_forward", layer_spec.feed_forward, dim, p)
+
+    def children(self):
+        return [c for c in (self.norm, self.mixer, self.feed_forward) if c is not None]
+
+    def first_norm(self):
+        return self.norm
+
+    def forward(self, x, ctx, line, writes_cache=True, next_norm=None):
+        left = ctx.normed.pop(id(self.norm), None)
+        if left is not None and left[1] is None:          # the layer before has left this norm's output
+            h = left[0]
+        else:
+            h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
+            self.norm.forward(x, h, ctx)
+        self.mixer.forward(h, x, ctx, line, writes_cache)
+        if self.feed_forward is not None:
+            self.feed_forward.forward(h, x, ctx)
+
+
 class StreamInput:
     """What `first_norm()` of a block that reads the residual stream itself hands to the layer before it: the
     place under which that layer may leave the stream in the compute dtype (ctx.normed[id(...)] = (h, None,

@@ -1,4 +1,4 @@
-"""Token embedding and the LM head.  The head is the embedding table itself
+"""Token embedding (optionally scaled, optionally with a sinusoidal position vector) and the LM head.  The head is the embedding table itself
 when tied (src/model.cpp:389-398); one copy on the device either way."""
 from ..ops import kernels
 from ..weights.loader import ParamSpec, place
@@ -7,25 +7,37 @@ from .base import Part, part
 
 @part("embedding", "token_embedding")
 class TokenEmbedding(Part):
-    """x[t] = float(table[token[t]]), no scaling (src/infer.cpp:454-475)."""
+    """x[t] = float(table[token[t]]) (src/infer.cpp:454-475), times `scale` (default 1), plus, with `sinusoid_base` b,
+    a position vector whose entry 2i is sin(p b^(-2i / width)) and whose entry 2i + 1 is the cosine of the same angle
+    (the frequencies are made in float64 and the angle is exact at every position)."""
 
     def __init__(self, spec, dim, prefix):
         super().__init__(spec, dim, prefix)
         self.vocab_size = int(spec.params["vocab_size"])
         self.tensor = self.prefix + str(spec.params.get("tensor", "weight"))      # the table's name in a folder
+        self.scale = float(spec.params.get("scale", 1.0))
+        self.sinusoid_base = spec.params.get("sinusoid_base")
         self.table = None
+        self.freq = None
 
     def param_specs(self):
         return [ParamSpec(self.tensor, (self.vocab_size, self.dim), init="embedding")]
 
     def load(self, get, compute_dtype, device):
         self.table = place(get(self.tensor), compute_dtype, device)
+        if self.sinusoid_base:
+            import torch
+            i = torch.arange((self.dim + 1) // 2, dtype=torch.float64)
+            base = torch.tensor(float(self.sinusoid_base), dtype=torch.float64)
+            self.freq = torch.pow(base, -2.0 * i / self.dim).to(device)
 
     def weight_bytes(self):
         return self.dim * self.table.element_size()          # one row per token
 
     def forward(self, tokens, x, ctx):
-        return kernels.embed(self.table, tokens, x)
+        if self.freq is None and self.scale == 1.0:
+            return kernels.embed(self.table, tokens, x)
+        return kernels.embed_sinusoid(self.table, tokens, ctx.tok_pos, self.freq, self.scale, x)
 
 
 @part("head", "lm_head")

@@ -1,9 +1,11 @@
 """Mixture of experts: `n_experts` small gated feed-forwards, of which a token uses the `top` whose router
 scores are largest.
 
-Router: s = softmax(W_router h) over all experts, in float32; the chosen experts' weights are their scores
-(`renormalize`: divided by their sum).  Expert: g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit),
-out = W_down (g sigmoid(alpha g) (u + 1)) (limit 0: no clamping).  The part's result is the weighted sum over
+Router: s = softmax(W_router h (+ a bias, the tensor `router_bias`)) over all experts, in float32; the chosen experts'
+weights are their scores (`renormalize`: divided by their sum; "chosen": the experts with the largest logits, weighted
+by the softmax over the chosen logits alone).  Expert: g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit),
+out = W_down (g sigmoid(alpha g) (u + up_shift)) (limit 0: no clamping; up_shift defaults to 1; alpha 1 and up_shift 0
+make silu(gate) * up).  The part's result is the weighted sum over
 a token's chosen experts, in the order of their scores.
 
 The experts' matrices are stacked at load ([E, F, D], [E, F, D], [E, D, F]); routing happens on the device
@@ -34,14 +36,17 @@ class MixtureOfExperts(Part):
         self.top = int(p["top"])
         self.limit = float(p.get("limit", 0.0) or 0.0)
         self.alpha = float(p.get("alpha", 1.0))
-        self.renormalize = bool(p.get("renormalize", False))
+        self.up_shift = float(p.get("up_shift", 1.0))
+        self.renormalize = p.get("renormalize", False)
+        self.renormalize = "chosen" if self.renormalize == "chosen" else bool(self.renormalize)
         self.expert_prefix = str(p.get("expert_prefix", "experts.%d."))
         self.names = {"router": "router", "gate": "gate", "up": "up", "down": "down"}
         self.names.update(p.get("tensors") or {})
+        self.router_bias = self.names.get("router_bias")           # a tensor's name, or no bias
         if not 0 < self.top <= self.n_experts or self.n_experts > kernels.MOE_MAX_EXPERTS:
             raise ValueError("mixture of experts: %d of %d experts is not offered (at most %d experts)"
                              % (self.top, self.n_experts, kernels.MOE_MAX_EXPERTS))
-        self.w_router = self.w_gate = self.w_up = self.w_down = None
+        self.w_router = self.w_gate = self.w_up = self.w_down = self.b_router = None
 
     def _expert(self, e, key):
         return self.prefix + (self.expert_prefix % e) + self.names[key]
@@ -49,6 +54,8 @@ class MixtureOfExperts(Part):
     def param_specs(self):
         D, F = self.dim, self.hidden
         out = [ParamSpec(self.prefix + self.names["router"], (self.n_experts, D), fan_in=D)]
+        if self.router_bias:
+            out.append(ParamSpec(self.prefix + self.router_bias, (self.n_experts,), init="bias"))
         for e in range(self.n_experts):
             out += [ParamSpec(self._expert(e, "gate"), (F, D), fan_in=D), ParamSpec(self._expert(e, "up"), (F, D), fan_in=D),
                     ParamSpec(self._expert(e, "down"), (D, F), fan_in=F)]
@@ -57,6 +64,8 @@ class MixtureOfExperts(Part):
     def load(self, get, compute_dtype, device):
         E = self.n_experts
         self.w_router = place(get(self.prefix + self.names["router"]), compute_dtype, device)
+        if self.router_bias:
+            self.b_router = get(self.prefix + self.router_bias).to(torch.float32).to(device).contiguous()
         self.w_gate = place(torch.stack([get(self._expert(e, "gate")) for e in range(E)]), compute_dtype, device)
         self.w_up = place(torch.stack([get(self._expert(e, "up")) for e in range(E)]), compute_dtype, device)
         self.w_down = place(torch.stack([get(self._expert(e, "down")) for e in range(E)]), compute_dtype, device)
@@ -76,12 +85,12 @@ class MixtureOfExperts(Part):
         wts = ws.get("moe.weights", (T, self.top), torch.float32)
         logits = ws.get("moe.logits", (T, self.n_experts), torch.float32)        # products exact, sums in float32
         self._gemm(ctx, h, self.w_router, logits, kernels.EPI_STORE_F32)
-        kernels.moe_select(logits, ids, wts, self.renormalize)
+        kernels.moe_select(logits, ids, wts, self.renormalize, bias=self.b_router)
         if T >= GROUPED_MIN_ROWS and kernels.can_moe_grouped(self.dim, self.hidden, h.dtype, T * self.top, self.n_experts):
             return kernels.moe_grouped(h, self.w_gate, self.w_up, self.w_down, ids, wts, self.limit, self.alpha, ws.get,
-                                       out, accumulate)
+                                       out, accumulate, up_shift=self.up_shift)
         mid = ws.get("moe.hidden", (T * self.top, self.hidden), h.dtype)
-        kernels.moe_pair_gate_up(h, self.w_gate, self.w_up, ids, self.limit, self.alpha, mid)
+        kernels.moe_pair_gate_up(h, self.w_gate, self.w_up, ids, self.limit, self.alpha, mid, up_shift=self.up_shift)
         kernels.moe_pair_down(mid, self.w_down, ids, wts, out, accumulate)
         return out
 

@@ -1,0 +1,168 @@
+"""Grouped-query attention without rotation, whose scores are shaped instead: every piece is a parameter and may
+be left out.
+
+Per token: q, k, v = W h (+ biases); RMS norms over the WHOLE query and key projections (all heads at once, plain
+weights; `projection_norm`); the query times 1 + coef ln(floor((p + 1) / every) + 1) at position p (`q_temp`);
+score = (q . k) * scale, capped as cap tanh(score / cap) (`softcap`), plus the position part's term by the
+distance (a slope a head); a window; a softmax whose denominator also holds exp(sink_h), a learned logit a head
+without key or value (`sink_logit`); the values of a layer with `value_blend` "later" are (1 - lam) v + lam v_first,
+v_first being the values that the layer with "first" made for the same token (lam a tensor), and the blended
+values are what the cache keeps.  Key and value heads may differ in size.
+
+The cache and the attention kernels are the library's grouped-query ones: a head is stored `pad` elements wide
+(the larger of key and value size, rounded up to 16, zeros behind), the output projection's columns are spread
+to that width at load, and scale * sqrt(pad) rides on the query, since the kernels divide by sqrt(pad)."""
+import math
+
+import torch
+
+from ..cache.manager import KVRequest
+from ..ops import kernels
+from ..weights.loader import ParamSpec, place
+from .attention import decode_splits, kv_tiles
+from .base import Part, build_part, part
+
+NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "out": "o_proj.weight",
+         "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "q_norm": "q_norm.weight",
+         "k_norm": "k_norm.weight", "sink": "sink", "blend": "value_blend"}
+
+
+@part("mixer", "shaped_attention")
+class ShapedAttention(Part):
+    prompt_tables = (kv_tiles,)
+
+    def __init__(self, spec, dim, prefix):
+        super().__init__(spec, dim, prefix)
+        p = spec.params
+        self.n_heads = int(p["n_heads"])
+        self.n_kv_heads = int(p.get("n_kv_heads") or self.n_heads)
+        self.key_dim = int(p["key_dim"])
+        self.value_dim = int(p.get("value_dim") or self.key_dim)
+        self.scale = float(p.get("scale") or self.key_dim ** -0.5)
+        self.softcap = float(p.get("softcap") or 0.0)
+        self.window = int(p.get("window", 0) or 0)
+        self.q_temp = tuple(p["q_temp"]) if p.get("q_temp") else None
+        self.projection_norm = bool(p.get("projection_norm", False))
+        self.eps = float(p.get("eps", 1e-6))
+        self.biases = bool(p.get("biases", False))
+        self.has_sink = bool(p.get("sink_logit", False))
+        self.value_blend = p.get("value_blend")
+        self.blend_name = str(p.get("blend_name", "blend"))
+        if self.value_blend not in (None, "first", "later"):
+            raise ValueError("value_blend %r is not None, 'first' or 'later'" % (self.value_blend,))
+        if self.n_heads % self.n_kv_heads:
+            raise ValueError("n_heads %d is no multiple of n_kv_heads %d" % (self.n_heads, self.n_kv_heads))
+        self.pad = (max(self.key_dim, self.value_dim) + 15) // 16 * 16
+        if self.pad > kernels.MAX_HEAD_DIM:
+            raise ValueError("heads of %d are not supported (at most %d)" % (self.pad, kernels.MAX_HEAD_DIM))
+        self.q_dim, self.k_dim, self.v_dim = self.n_heads * self.key_dim, self.n_kv_heads * self.key_dim, self.n_kv_heads * self.value_dim
+        if (self.q_dim + self.k_dim + self.v_dim) * 4 > 64 * 1024:
+            raise ValueError("a token's queries, keys and values (%d numbers) are more than the packing kernel holds"
+                             % (self.q_dim + self.k_dim + self.v_dim))
+        self.names = dict(NAMES)
+        self.names.update(p.get("tensors") or {})
+        self.position = build_part("position", p["position"], dim, prefix) if p.get("position") else None
+        self.wqkv = self.wo = self.bias = self.w_qn = self.w_kn = self.sink = self.lam = None
+
+    def children(self):
+        return [self.position] if self.position is not None else []
+
+    def _n(self, key):
+        return self.prefix + self.names[key]
+
+    def param_specs(self):
+        D = self.dim
+        out = [ParamSpec(self._n("q"), (self.q_dim, D), fan_in=D), ParamSpec(self._n("k"), (self.k_dim, D), fan_in=D),
+               ParamSpec(self._n("v"), (self.v_dim, D), fan_in=D),
+               ParamSpec(self._n("out"), (D, self.n_heads * self.value_dim), fan_in=self.n_heads * self.value_dim)]
+        if self.biases:
+            out += [ParamSpec(self._n("q_bias"), (self.q_dim,), init="bias"), ParamSpec(self._n("k_bias"), (self.k_dim,), init="bias"),
+                    ParamSpec(self._n("v_bias"), (self.v_dim,), init="bias")]
+        if self.projection_norm:
+            out += [ParamSpec(self._n("q_norm"), (self.q_dim,), init="norm"), ParamSpec(self._n("k_norm"), (self.k_dim,), init="norm")]
+        if self.has_sink:
+            out.append(ParamSpec(self._n("sink"), (self.n_heads,), init="embedding"))
+        if self.value_blend is not None:
+            # the first blending layer's number is in the folder and is not used
+            out.append(ParamSpec(self._n("blend"), (), init="fraction"))
+        return out
+
+    def load(self, get, compute_dtype, device):
+        def f32(key):
+            return get(self._n(key)).to(torch.float32).reshape(-1).to(device).contiguous()
+        self.wqkv = place(torch.cat([get(self._n("q")), get(self._n("k")), get(self._n("v"))], dim=0), compute_dtype, device)
+        wo = get(self._n("out"))
+        if self.pad != self.value_dim:                    # the attention's result is `pad` wide a head, zeros behind
+            spread = torch.zeros((self.dim, self.n_heads, self.pad), dtype=wo.dtype)
+            spread[:, :, :self.value_dim] = wo.reshape(self.dim, self.n_heads, self.value_dim)
+            wo = spread.reshape(self.dim, self.n_heads * self.pad)
+        self.wo = place(wo, compute_dtype, device)
+        self.bias = torch.cat([f32("q_bias"), f32("k_bias"), f32("v_bias")]).contiguous() if self.biases else None
+        self.w_qn, self.w_kn = (f32("q_norm"), f32("k_norm")) if self.projection_norm else (None, None)
+        self.sink = f32("sink") if self.has_sink else None
+        self.lam = f32("blend") if self.value_blend == "later" else None
+
+    def weight_bytes(self):
+        return (self.wqkv.numel() + self.wo.numel()) * self.wqkv.element_size()
+
+    def cache_request(self):
+        return KVRequest(self.n_kv_heads, self.pad, self.window, 0)
+
+    def row_elements(self):
+        return max(self.q_dim + self.k_dim + self.v_dim, self.n_heads * self.pad)
+
+    def describe(self, compute_dtype):
+        what = "shaped attention, %d heads in %d groups, keys of %d and values of %d in heads of %d%s" % (
+            self.n_heads, self.n_kv_heads, self.key_dim, self.value_dim, self.pad,
+            ", window %d" % self.window if self.window else "")
+        if compute_dtype != torch.bfloat16:
+            return what + ": float32-arithmetic kernels", False
+        if self.pad in kernels.MFMA_HEAD_DIMS:
+            return what + ": matrix-core kernels", False
+        return what + ": float32-arithmetic kernels on bfloat16 storage (the matrix-core kernels take head sizes " \
+                      "of 16 to 128 in steps of 16, not %d): correct, several times slower" % self.pad, True
+
+    @property
+    def score_bias(self):
+        return getattr(self.position, "score_bias", None)
+
+    def forward(self, h, x, ctx, line, writes_cache=True):
+        T = h.shape[0]
+        act, ws = h.dtype, ctx.ws
+        H, G, P = self.n_heads, self.n_kv_heads, self.pad
+        if self.position is not None and ctx.max_position >= self.position.n_positions:
+            raise ValueError("position %d is beyond the %d distances the score table holds"
+                             % (ctx.max_position, self.position.n_positions))
+        prefill = ctx.mode == "prefill"
+        qkv = ws.get("attn.qkv", (T, self.q_dim + self.k_dim + self.v_dim), torch.float32)
+        self._gemm(ctx, h, self.wqkv, qkv, kernels.EPI_STORE_F32)
+        q = ws.get("attn.q", (T, H * P), act)
+        group = ctx.cache.group_of(line)
+        k_pages, v_pages = group.line_pages(line)
+        kst = vst = seq_tile0 = None
+        if prefill:
+            tiles = ctx.tables["kv_tiles"]
+            seq_tile0, n_tiles = tiles["seq_tile0"], tiles["n_tiles"]
+            kst = ws.get("attn.stage.k", (n_tiles, G, kernels.PAGE, P), act)
+            vst = ws.get("attn.stage.v", (n_tiles, G, P, kernels.PAGE), act)
+        v_first, blend = None, 0
+        if self.value_blend is not None:
+            # the first blending layer of a step leaves its values here for the later ones of the same step
+            v_first = ws.get("attn.blend." + self.blend_name, (T, self.v_dim), torch.float32)
+            blend = 1 if self.value_blend == "first" else 2
+        kernels.qkv_pack(qkv, self.bias, self.w_qn, self.w_kn, self.eps, self.q_temp, self.scale * math.sqrt(P), v_first,
+                         blend, self.lam, q, kst, vst, seq_tile0, k_pages if writes_cache else None,
+                         v_pages if writes_cache else None, group.table, group.ring_pages, ctx.tok_seq, ctx.tok_pos,
+                         ctx.seq_slot, ctx.seq_len, H, G, self.key_dim, self.value_dim, P)
+        o = ws.get("attn.o", (T, H * P), act)
+        if prefill:
+            kernels.attn_prefill(q, kst, vst, o, ctx.cu_seqlens, seq_tile0, ctx.tok_seq, ctx.tok_pos, H, G, P, self.window,
+                                 tiles.get("tile_order"), score_bias=self.score_bias, softcap=self.softcap,
+                                 sink_logit=self.sink)
+        else:
+            n_splits = decode_splits(H, G, P, T, min(group.ring_pages, ctx.pages_bucket), ctx.ragged)
+            partial = ws.get("attn.partial", (kernels.attn_decode_workspace_floats(T, H, P, n_splits),), torch.float32)
+            kernels.attn_decode(q, k_pages, v_pages, group.table, group.ring_pages, ctx.seq_slot, ctx.seq_len, o, partial,
+                                H, G, P, self.window, n_splits, step_max_len=ctx.step_max_len, seq_order=ctx.seq_order,
+                                score_bias=self.score_bias, softcap=self.softcap, sink_logit=self.sink)
+        self._gemm(ctx, o, self.wo, x, kernels.EPI_ADD_F32)

@@ -39,19 +39,22 @@ class SwiGLU(Part):
         if self.activation not in ACTIVATIONS:
             raise ValueError("feed-forward activation %r is not offered (%s)" % (self.activation, ", ".join(ACTIVATIONS)))
         self.gated = ACTIVATIONS[self.activation]          # the GEMM epilogue that applies it
+        # the tensors' names behind the part's prefix (parameter `tensors`: {gate, up, down})
+        self.names = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+        self.names.update(spec.params.get("tensors") or {})
         self.w_gate_up = None
         self.w_down = None
 
     def param_specs(self):
         D, H = self.dim, self.hidden
-        return [ParamSpec(self.prefix + "gate_proj.weight", (H, D), fan_in=D),
-                ParamSpec(self.prefix + "up_proj.weight", (H, D), fan_in=D),
-                ParamSpec(self.prefix + "down_proj.weight", (D, H), fan_in=H)]
+        return [ParamSpec(self.prefix + self.names["gate"], (H, D), fan_in=D),
+                ParamSpec(self.prefix + self.names["up"], (H, D), fan_in=D),
+                ParamSpec(self.prefix + self.names["down"], (D, H), fan_in=H)]
 
     def load(self, get, compute_dtype, device):
-        gu = interleave_gate_up(get(self.prefix + "gate_proj.weight"), get(self.prefix + "up_proj.weight"))
+        gu = interleave_gate_up(get(self.prefix + self.names["gate"]), get(self.prefix + self.names["up"]))
         self.w_gate_up = place(gu, compute_dtype, device)
-        self.w_down = place(get(self.prefix + "down_proj.weight"), compute_dtype, device)
+        self.w_down = place(get(self.prefix + self.names["down"]), compute_dtype, device)
 
     def weight_bytes(self):
         return 3 * self.hidden * self.dim * self.w_down.element_size()

@@ -32,7 +32,7 @@ class WeightsError(ValueError):
 class ParamSpec:
     """A tensor a part needs: full name in the folder, shape, and how random
     weights are drawn for it ('linear': U(-1/sqrt(fan_in), 1/sqrt(fan_in));
-    'norm': 1 + U(-0.1, 0.1); 'embedding': N(0, 1); 'zeros')."""
+    'norm': 1 + U(-0.1, 0.1); 'embedding': N(0, 1); 'bias': U(-0.5, 0.5); 'fraction': U(0.1, 0.9); 'zeros')."""
     name: str
     shape: Tuple[int, ...]
     init: str = "linear"

@@ -71,6 +71,10 @@ def random_values(name, shape, init, fan_in, seed, device="cpu"):
         elif init == "embedding":
             u2 = _uniform01(key, start, n, 1, device)
             v = torch.sqrt(-2.0 * torch.log(u + (1.0 / (1 << 24)))) * torch.cos((2.0 * math.pi) * u2)
+        elif init == "bias":
+            v = (u * 2.0 - 1.0) * 0.5
+        elif init == "fraction":
+            v = 0.1 + u * 0.8
         elif init == "zeros":
             v = torch.zeros(n, dtype=torch.float32, device=device)
         else:
