@@ -8,7 +8,7 @@ shape with its window of 4,096 positions and prompts of 6,000 tokens).
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--dtype bf16|fp32] [--shape NAME]
                     [--prompt-len N] [--prefill-len N] [--batch B] [--points B,B] [--no-prefill]
                     [--kernels] [--ragged] [--sweep]
-    python bench.py --design situlorn [--sizes 2048,4096] [--kernels] [--steps K] [--warmup W]
+    python bench.py --design situlorn|gedunex [--sizes 2048,4096] [--kernels] [--steps K] [--warmup W]
 
 --kernels adds the time of every kernel of a decode step and of a prompt step, each taken alone at the
 shape's sizes (src/test.cpp:340-405 times single kernels so), with its rate against the peak;
@@ -18,8 +18,10 @@ shape's sizes (src/test.cpp:340-405 times single kernels so), with its rate agai
 --design situlorn measures another model design beside the closest one the library has: four layers of the
 Situlorn design (latent attention with and without a window, one layer on another's keys, dense PolyNorm and
 mixture-of-experts feed-forwards) and four Llama layers of the same width and about the same weights, each a
-prompt of --prefill-len tokens and decode steps at --batch; with --kernels every kernel of both alone.  The default
-workload and its line stay as they are.
+prompt of --prefill-len tokens and decode steps at --batch; with --kernels every kernel of both alone.  --design
+gedunex does the same for four layers of the Gedunex design (three shaped attentions under a window and one mLSTM,
+dense and mixture-of-experts feed-forwards) beside the Situlorn and the Llama layers.  The default workload and its
+line stay as they are.
 
 A step is one decode step as generation does it: the step function for a batch
 of sequences (one token each, from the cache), greedy sampling on the device
@@ -110,7 +112,9 @@ def measured_peaks(torch, dtype):
 KERNEL_FACES = ("embed", "rmsnorm", "gemm", "gemm_norm", "gemm_norm_qkv_rope", "gemm_add_norm", "gemm_add_emit", "gemm_partial",
                 "gemm_chain", "gemm_chain_qkv_rope", "rope_kv_write", "rope_kv_write_tiles", "attn_prefill",
                 "attn_decode", "sink_store", "attn_sink_mix", "argmax", "cast", "norm_add", "polynorm", "head_matmul",
-                "latent_pack", "moe_route", "moe_pair_gate_up", "moe_pair_down", "moe_grouped")
+                "latent_pack", "moe_route", "moe_select", "moe_pair_gate_up", "moe_pair_down", "moe_grouped", "embed_sinusoid",
+                "qkv_pack", "mlstm_scan")
+FP32_FACES = ("mlstm_scan",)     # kernels of float32 multiply-adds whatever the model's dtype: priced against that peak
 
 
 def record_kernel_calls(run):
@@ -187,6 +191,20 @@ def kernel_cost(name, a, kw, kv_tokens, torch):
         return "polynorm %dx%d" % tuple(a[0].shape), nbytes(a[0], a[3]), 0.0
     if name == "cast":
         return "cast %d" % a[0].numel(), nbytes(a[0], a[1]), 0.0
+    if name == "embed_sinusoid":
+        return "embed_sinusoid %d" % a[1].shape[0], 2 * nbytes(a[5]), 0.0
+    if name == "moe_select":
+        return "moe_select %d tokens" % a[0].shape[0], nbytes(a[0], a[1], a[2]), 0.0
+    if name == "qkv_pack":
+        qkv, q_out = a[0], a[10]
+        T = qkv.shape[0]
+        n_kv, pad = a[23], a[26]
+        return "qkv_pack %d tokens" % T, nbytes(qkv, q_out) + 2 * T * n_kv * pad * q_out.element_size() * (2 if a[11] is not None else 1), 0.0
+    if name == "mlstm_scan":
+        proj, state, seq_slot, out = a[0], a[4], a[6], a[7]
+        H, d, dv = a[8], a[9], a[10]
+        T, B = proj.shape[0], seq_slot.shape[0]
+        return "mlstm_scan %d tokens" % T, nbytes(proj, out) + 2 * B * H * (d * dv + d + 1) * 4, 4.0 * T * H * d * dv
     if name == "moe_route":
         return "moe_route %d tokens" % a[0].shape[0], nbytes(a[0], a[1]), 2.0 * a[0].shape[0] * a[1].numel()
     if name in ("moe_pair_gate_up", "moe_pair_down", "moe_grouped"):
@@ -245,7 +263,8 @@ def time_kernel_groups(calls, kv_tokens, torch, dtype, reps=5):
         us = total / reps / n * 1e3
         gbs = g["bytes"] / us / 1e3
         tfs = g["flops"] / us / 1e6
-        frac_hbm, frac_mfma = gbs * 1e9 / HBM_PEAK, tfs * 1e12 / FLOP_PEAK[dtype]
+        peak = FLOP_PEAK["fp32"] if label.split(" ")[0] in FP32_FACES else FLOP_PEAK[dtype]
+        frac_hbm, frac_mfma = gbs * 1e9 / HBM_PEAK, tfs * 1e12 / peak
         bound = "hbm" if frac_hbm >= frac_mfma else "mfma"
         out[label] = {"calls": n, "us": round(us, 2), "GB/s": round(gbs, 1), "TFLOP/s": round(tfs, 2),
                       "bound": bound, "frac": round(max(frac_hbm, frac_mfma), 4)}
@@ -275,6 +294,21 @@ def situlorn_config(width, n_layers=4):
             "layers": [pattern[i % 4] for i in range(n_layers)]}
 
 
+def gedunex_config(width, n_layers=4):
+    """Layers of the Gedunex design at a real model's sizes: attention heads of 128 in groups of four under a window
+    of 1,024, mLSTM heads of 128 x 256, the feed-forwards of situlorn_config's sizes."""
+    heads = width // 128
+    attn = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0,
+            "mask": {"size": 1024}, "q_temp": {"coef": 0.1, "every": 1024}, "v_mix": True}
+    rec = {"heads": max(1, width // 256), "dim": 128, "vdim": 256, "gate_cap": 15.0}
+    dense = {"kind": "dense", "ff": width * 7 // 2}
+    moe = {"kind": "moe", "expert": {"ff": width // 2}, "router": {"experts": 32, "top": 4}}
+    pattern = [{"type": "attention", "mixer": attn, "mlp": dense}, {"type": "attention", "mixer": attn, "mlp": moe},
+               {"type": "mlstm", "mixer": rec, "mlp": moe}, {"type": "attention", "mixer": attn, "mlp": dense}]
+    return {"architecture": "Gedunex", "vocab": 32000, "width": width, "norm": {"eps": 1e-5},
+            "embedding": {"scale": float(width) ** 0.5}, "layers": [pattern[i % 4] for i in range(n_layers)]}
+
+
 def llama_config(width, n_layers=4):
     return {"architectures": ["LlamaForCausalLM"], "hidden_size": width, "intermediate_size": width * 7 // 2,
             "num_hidden_layers": n_layers, "num_attention_heads": width // 128, "num_key_value_heads": width // 512,
@@ -293,7 +327,9 @@ def bench_design(args):
     sampler = Sampler(0)
     out = {}
     for width in [int(w) for w in args.sizes.split(",") if w]:
-        for design, cfg in (("situlorn", situlorn_config(width)), ("llama", llama_config(width))):
+        own = ("gedunex", gedunex_config(width)) if args.design == "gedunex" else ("situlorn", situlorn_config(width))
+        beside = (("situlorn", situlorn_config(width)),) if args.design == "gedunex" else ()
+        for design, cfg in (own,) + beside + (("llama", llama_config(width)),):
             model = Model.random(cfg, seed=0, dtype=dtype, device="cuda:0")
             V = model.vocab_size
             engine = Engine(model, max_tokens=B * (PROMPT + args.steps + args.warmup + 128) + T + 64, max_batch=B)
@@ -361,7 +397,8 @@ def bench_design(args):
             out["%s_%d" % (design, width)] = r
             del engine, model
             torch.cuda.empty_cache()
-    print(json.dumps({"metric": "prompt and decode steps of 4 Situlorn layers beside 4 Llama layers of equal width",
+    print(json.dumps({"metric": "prompt and decode steps of 4 %s layers beside 4 Llama layers of equal width"
+                                % args.design.capitalize(),
                       "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype,
                       "data": "synthetic: seeded random weights and token ids", "sizes": out}), flush=True)
     return 0
@@ -395,7 +432,7 @@ def main():
     ap.add_argument("--context", type=int, default=0,
                     help="the reference's -T: past this many positions two attention sinks and the last "
                          "<context> - 2 positions are attended to (0: the shape's own window, if any)")
-    ap.add_argument("--design", default="", choices=["", "situlorn"],
+    ap.add_argument("--design", default="", choices=["", "situlorn", "gedunex"],
                     help="measure layers of this design beside Llama layers of equal width instead of the default workload")
     ap.add_argument("--sizes", default="2048,4096", help="widths for --design")
     args = ap.parse_args()

@@ -50,7 +50,7 @@ __global__ void embed_sinusoid_kernel(const T* __restrict__ table, const int* __
     return;
   }
   const T* row = table + (size_t)tok * D;
-  const double p = (double)positions[t];
+  const double p = freq != nullptr ? (double)positions[t] : 0.0;      // no positions are given without frequencies
   for (int i = threadIdx.x; i < D; i += blockDim.x) {
     float v = to_f32(row[i]) * scale;
     if (freq != nullptr) {
