@@ -113,8 +113,8 @@ KERNEL_FACES = ("embed", "rmsnorm", "gemm", "gemm_norm", "gemm_norm_qkv_rope", "
                 "gemm_chain", "gemm_chain_qkv_rope", "rope_kv_write", "rope_kv_write_tiles", "attn_prefill",
                 "attn_decode", "sink_store", "attn_sink_mix", "argmax", "cast", "norm_add", "polynorm", "head_matmul",
                 "latent_pack", "moe_route", "moe_select", "moe_pair_gate_up", "moe_pair_down", "moe_grouped", "embed_sinusoid",
-                "qkv_pack", "mlstm_scan")
-FP32_FACES = ("mlstm_scan",)     # kernels of float32 multiply-adds whatever the model's dtype: priced against that peak
+                "qkv_pack", "mlstm_scan", "mlstm_chunks")
+FP32_FACES = ("mlstm_scan", "mlstm_chunks")     # kernels of float32 multiply-adds whatever the model's dtype: priced against that peak
 
 
 def record_kernel_calls(run):
@@ -205,6 +205,14 @@ def kernel_cost(name, a, kw, kv_tokens, torch):
         H, d, dv = a[8], a[9], a[10]
         T, B = proj.shape[0], seq_slot.shape[0]
         return "mlstm_scan %d tokens" % T, nbytes(proj, out) + 2 * B * H * (d * dv + d + 1) * 4, 4.0 * T * H * d * dv
+    if name == "mlstm_chunks":
+        proj, state, seq_slot, out = a[0], a[4], a[8], a[9]
+        H, d, dv, chunk = a[10], a[11], a[12], a[17]
+        T, B = proj.shape[0], seq_slot.shape[0]
+        # per token and head: the scores against a chunk's earlier tokens (half a chunk on average), their mix of the
+        # values, the query on the carried state and the token's share of the state's update
+        per_token = 2.0 * d * min(chunk, max(T // B, 1)) / 2 + 2.0 * dv * min(chunk, max(T // B, 1)) / 2 + 4.0 * d * dv
+        return "mlstm_chunks %d tokens" % T, nbytes(proj, out) + 2 * nbytes(a[5]) + 2 * B * H * (d * dv + d + 1) * 4, T * H * per_token
     if name == "moe_route":
         return "moe_route %d tokens" % a[0].shape[0], nbytes(a[0], a[1]), 2.0 * a[0].shape[0] * a[1].numel()
     if name in ("moe_pair_gate_up", "moe_pair_down", "moe_grouped"):

@@ -105,15 +105,17 @@ def test_packing_kernel(dtype, H, G, d, dv, temp, blend):
         assert torch.allclose(v_first.cpu().to(F64), v.reshape(T, V), rtol=0, atol=1e-6)
 
 
+@pytest.mark.parametrize("how", ["token by token", "chunks"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,d,dv,cap", [(1, 4, 4, 3.0), (2, 8, 6, 4.0), (3, 20, 7, 0.0), (1, 64, 200, 30.0), (2, 128, 256, 15.0),
-                                        (5, 3, 5, 2.0)])
-def test_recurrence_kernel(dtype, H, d, dv, cap):
-    """Two sequences and a padding row: the first pieces of the texts as a step of whole prompts, then single tokens,
-    against the plain recurrence over the whole texts; the state left behind against the plain one's."""
+                                        (5, 3, 5, 2.0), (1, 40, 70, 6.0)])
+def test_recurrence_kernel(dtype, H, d, dv, cap, how):
+    """Two sequences and a padding row: the first pieces of the texts as a step of whole prompts (one of them longer than
+    two chunks), then single tokens, against the plain recurrence over the whole texts; the state left behind against the
+    plain one's.  Both kernels: the one that walks token by token and the one that takes a chunk at a time."""
     from yalm_amd.ops import kernels
     D = H * dv
-    lens = [37, 5]
+    lens = [167, 5]
     g = gen(H * 100 + d)
     sc = 1.0 / np.sqrt(D)
     w = {"m." + k: torch.randn(s, generator=g, dtype=F64) * sc for k, s in
@@ -133,17 +135,24 @@ def test_recurrence_kernel(dtype, H, d, dv, cap):
     def step(rows, cu, seq_slot):
         proj = f32(torch.cat(rows) @ W_in.T)
         out = torch.empty(proj.shape[0], H * dv, dtype=dtype, device=DEV)
-        kernels.mlstm_scan(proj, f32(w["m.i.b"]), f32(w["m.f.b"]), f32(w["m.norm"]), state, i32(cu), i32(seq_slot), out, H, d, dv,
-                           d ** -0.5, cap, P.MLSTM_FLOOR, 1e-5)
+        if how == "chunks":
+            raw = torch.full((proj.shape[0], H * dv), float("nan"), dtype=torch.float32, device=DEV)
+            nm = torch.full((len(seq_slot), H * (d + 1)), float("nan"), dtype=torch.float32, device=DEV)
+            kernels.mlstm_chunks(proj, f32(w["m.i.b"]), f32(w["m.f.b"]), f32(w["m.norm"]), state, raw, nm, i32(cu), i32(seq_slot),
+                                 out, H, d, dv, d ** -0.5, cap, P.MLSTM_FLOOR, 1e-5, 64 if len(rows[0]) > 1 else 16)
+        else:
+            kernels.mlstm_scan(proj, f32(w["m.i.b"]), f32(w["m.f.b"]), f32(w["m.norm"]), state, i32(cu), i32(seq_slot), out, H, d,
+                               dv, d ** -0.5, cap, P.MLSTM_FLOOR, 1e-5)
         return out.float().cpu().to(F64)
     got = [[], []]
-    out = step([hs[0][:30], hs[1][:2]], [0, 30, 32], slots)
-    got[0].append(out[:30]); got[1].append(out[30:])
+    out = step([hs[0][:160], hs[1][:2]], [0, 160, 162], slots)
+    got[0].append(out[:160]); got[1].append(out[160:])
     for t in range(7):                             # one token each, a padding row between them; the short text ends first
-        rows, ss = [hs[0][30 + t:31 + t], torch.zeros(1, D, dtype=F64)], [slots[0], -1]
+        rows, ss = [hs[0][160 + t:161 + t], torch.zeros(1, D, dtype=F64)], [slots[0], -1]
         if 2 + t < lens[1]:
             rows.append(hs[1][2 + t:3 + t]); ss.append(slots[1])
         out = step(rows, list(range(len(rows) + 1)), ss)
+        assert float(out[1].abs().max()) == 0.0      # the padding row
         got[0].append(out[0:1])
         if 2 + t < lens[1]:
             got[1].append(out[2:3])

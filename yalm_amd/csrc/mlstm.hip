@@ -37,8 +37,12 @@ __global__ __launch_bounds__(ML_THREADS) void mlstm_scan_kernel(
   __shared__ float gate[3];                       // keep, take, m
   const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
   const int slot = seq_slot[b];
-  if (slot < 0 || slot >= n_slots) return;        // a padding row: the whole workgroup leaves
   const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
+  if (slot < 0 || slot >= n_slots) {              // a padding row: zeros, and the whole workgroup leaves
+    for (int t = t0; t < t1; ++t)
+      for (int c = tid; c < dv; c += ML_THREADS) out[(size_t)t * H * dv + h * dv + c] = from_f32<T>(0.f);
+    return;
+  }
   if (t1 <= t0) return;
   const int per = d * dv + d + 1;
   float* st = state + ((size_t)slot * H + h) * per;
@@ -111,7 +115,287 @@ __global__ __launch_bounds__(ML_THREADS) void mlstm_scan_kernel(
 }
 
 LdsAllowance ml_allow_f32, ml_allow_bf16;
+
+// ---------------------------------------------------------------------------------------------------------------
+// The same recurrence a chunk of L tokens at a time, on the matrix cores in float32 (v_mfma_f32_16x16x4_f32: products
+// and sums of 32-bit floats).  With b_t the sum of the log forget gates from the chunk's start to t, w_s = i_s - b_s,
+// g_t = max(m0, max_{s<=t} w_s) and m0 the running maximum before the chunk, the running maximum at t is b_t + g_t and
+//   S_t^T q_t = exp(m0 - g_t) S0^T q_t + sum_{s<=t} exp(w_s - g_t) (k_s . q_t) v_s          (n_t . q_t likewise),
+// every exponent at most 0; the state behind the chunk is exp(m0 - g_L) S0 + sum_s exp(w_s - g_L) k_s v_s^T.
+// A workgroup owns 64 columns of one (sequence, head): the columns of S do not depend on each other, so a head's
+// dv / 64 workgroups run side by side (each forms the scores q . k again).  It leaves num / den of every token in
+// `raw` (float32 [T, H dv]); the norm over a head's dv values, which spans workgroups, is mlstm_finish_kernel's, and
+// so is putting n and m back (they go through `nm`, [B, H, d + 1], because a head's other workgroups may still have to
+// read the old ones).
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+constexpr int DVS = 64;                           // columns of S a workgroup owns
+constexpr int VROW = DVS + 16;                    // LDS row strides (floats)
+constexpr float NEVER = -3.0e38f;
+
+template <int L>
+__host__ __device__ constexpr size_t chunk_lds_floats(int d16) {
+  return (size_t)d16 * VROW + 2 * (size_t)L * (d16 + 4) + (size_t)L * VROW + (size_t)L * (L + 4) + d16 + 8 * L;
+}
+
+template <int L>
+__global__ __launch_bounds__(ML_THREADS) void mlstm_chunk_kernel(
+    const float* __restrict__ proj, const float* __restrict__ b_i, const float* __restrict__ b_f,
+    float* __restrict__ state, float* __restrict__ nm, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ seq_slot, float* __restrict__ raw, int H, int d, int dv, float q_scale, float cap,
+    float floor_, int n_slots) {
+  extern __shared__ float lds[];
+  const int d16 = (d + 15) / 16 * 16, QROW = d16 + 4, PROW = L + 4;
+  float* Ss = lds;                                // [d16][VROW]
+  float* Qs = Ss + (size_t)d16 * VROW;            // [L][QROW]
+  float* Ks = Qs + (size_t)L * QROW;              // [L][QROW]
+  float* Vs = Ks + (size_t)L * QROW;              // [L][VROW]
+  float* Ps = Vs + (size_t)L * VROW;              // [L][PROW]
+  float* nv = Ps + (size_t)L * PROW;              // [d16]
+  float* wv = nv + d16;                           // [L] w_s
+  float* gv = wv + L;                             // [L] g_t
+  float* ev = gv + L;                             // [L] exp(m0 - g_t)
+  float* mv = ev + L;                             // [L] the running maximum at t
+  float* cv = mv + L;                             // [L] exp(w_s - g_L)
+  float* rs = cv + L;                             // [L] sum_s P[t][s]
+  float* qn = rs + L;                             // [L] q_t . n0
+  float* bv = qn + L;                             // [L] b_t
+  const int slice = blockIdx.x, h = blockIdx.y, b = blockIdx.z, tid = threadIdx.x;
+  const int wave = tid / WAVE, lane = tid % WAVE, lr = lane % 16, lq = lane / 16;
+  const int slot = seq_slot[b];
+  if (slot < 0 || slot >= n_slots) return;        // a padding row (mlstm_finish_kernel writes its zeros)
+  const int t_begin = cu_seqlens[b], t_end = cu_seqlens[b + 1];
+  if (t_end <= t_begin) return;
+  const int per = d * dv + d + 1;
+  float* st = state + ((size_t)slot * H + h) * per;
+  const int col0 = slice * DVS;
+  for (int i = tid; i < d16 * DVS; i += ML_THREADS) {
+    const int k = i / DVS, c = i % DVS;
+    Ss[k * VROW + c] = k < d && col0 + c < dv ? st[(size_t)k * dv + col0 + c] : 0.f;
+  }
+  for (int k = tid; k < d16; k += ML_THREADS) nv[k] = k < d ? st[(size_t)d * dv + k] : 0.f;
+  float m0 = st[(size_t)d * dv + d];
+  const int N = 2 * H * d + 2 * H * dv + 2 * H;
+  constexpr int RT = L / 16;                      // row tiles of a chunk
+
+  for (int t0 = t_begin; t0 < t_end; t0 += L) {
+    const int n_valid = min(L, t_end - t0);
+    __syncthreads();                              // the chunk before is done with Qs, Ks, Vs, Ps and the vectors
+    for (int i = tid; i < L * d16; i += ML_THREADS) {
+      const int t = i / d16, k = i % d16;
+      const bool ok = t < n_valid && k < d;
+      const float* row = proj + (size_t)(t0 + t) * N;
+      Qs[t * QROW + k] = ok ? row[h * d + k] * q_scale : 0.f;
+      Ks[t * QROW + k] = ok ? row[H * d + h * d + k] : 0.f;
+    }
+    for (int i = tid; i < L * DVS; i += ML_THREADS) {
+      const int t = i / DVS, c = i % DVS;
+      Vs[t * VROW + c] = t < n_valid && col0 + c < dv ? proj[(size_t)(t0 + t) * N + 2 * H * d + h * dv + col0 + c] : 0.f;
+    }
+    if (wave == 0) {                              // the gates of the chunk: sums and maxima along it, a lane a token
+      float f = 0.f, zi = NEVER;
+      if (lane < n_valid) {
+        const float* row = proj + (size_t)(t0 + lane) * N + 2 * H * d + 2 * H * dv;
+        zi = row[h] + b_i[h];
+        float zf = row[H + h] + b_f[h];
+        if (cap > 0.f) {
+          zi = cap * tanhf(zi / cap);
+          zf = cap * tanhf(zf / cap);
+        }
+        f = log_sigmoid(zf);
+      }
+      float bsum = f;
+#pragma unroll
+      for (int o = 1; o < WAVE; o <<= 1) {
+        const float up = __shfl_up(bsum, o, WAVE);
+        if (lane >= o) bsum += up;
+      }
+      const float w = lane < n_valid ? zi - bsum : NEVER;
+      float a = w;
+#pragma unroll
+      for (int o = 1; o < WAVE; o <<= 1) {
+        const float up = __shfl_up(a, o, WAVE);
+        if (lane >= o) a = fmaxf(a, up);
+      }
+      const float g = fmaxf(m0, a);
+      const float gl = __shfl(g, n_valid - 1, WAVE);
+      if (lane < L) {
+        wv[lane] = w;
+        gv[lane] = g;
+        ev[lane] = expf(m0 - g);
+        mv[lane] = bsum + g;
+        bv[lane] = bsum;
+        cv[lane] = lane < n_valid ? expf(w - gl) : 0.f;
+      }
+    }
+    __syncthreads();
+    // scores: P[t][s] = (q_t . k_s) exp(w_s - g_t) for s <= t; a wave a tile of 16 tokens
+    if (wave < RT) {
+      for (int c = 0; c < RT; ++c) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        if (c <= wave) {
+          const float* qa = Qs + (wave * 16 + lr) * QROW + lq;
+          const float* kb = Ks + (c * 16 + lr) * QROW + lq;
+          for (int k0 = 0; k0 < d16; k0 += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[k0], kb[k0], acc, 0, 0, 0);
+        }
+        const int s_ = c * 16 + lr;
+        const float ws = wv[s_];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int t = wave * 16 + lq * 4 + v;
+          Ps[t * PROW + s_] = s_ <= t ? acc[v] * expf(ws - gv[t]) : 0.f;
+        }
+      }
+    }
+    __syncthreads();
+    if (tid < L) {
+      float a = 0.f;
+      for (int s_ = 0; s_ <= tid; ++s_) a += Ps[tid * PROW + s_];
+      rs[tid] = a;
+    } else if (tid >= WAVE && tid < WAVE + L) {
+      const int t = tid - WAVE;
+      float a = 0.f;
+      for (int k = 0; k < d16; ++k) a = fmaf(Qs[t * QROW + k], nv[k], a);
+      qn[t] = a;
+    }
+    __syncthreads();
+    // the tokens' results: P V + exp(m0 - g_t) Q S0, over the denominator
+    if (wave < RT) {
+      for (int c = 0; c < DVS / 16; ++c) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+        const float* pa = Ps + (wave * 16 + lr) * PROW + lq;
+        const float* vb = Vs + lq * VROW + c * 16 + lr;
+        for (int s0 = 0; s0 < (wave + 1) * 16; s0 += 4)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[s0], vb[s0 * VROW], acc, 0, 0, 0);
+        const float* qa = Qs + (wave * 16 + lr) * QROW + lq;
+        const float* sb = Ss + lq * VROW + c * 16 + lr;
+        for (int k0 = 0; k0 < d16; k0 += 4)
+          acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[k0], sb[k0 * VROW], acc2, 0, 0, 0);
+        const int col = col0 + c * 16 + lr;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int t = wave * 16 + lq * 4 + v;
+          if (t < n_valid && col < dv) {
+            const float e = ev[t];
+            const float den = fmaxf(fabsf(fmaf(e, qn[t], rs[t])), expf(-mv[t])) + floor_;
+            raw[(size_t)(t0 + t) * H * dv + h * dv + col] = fmaf(e, acc2[v], acc[v]) / den;
+          }
+        }
+      }
+    }
+    __syncthreads();
+    // the state behind the chunk: exp(m0 - g_L) S0 + (c K)^T V; wave w owns the column tile w of every row tile
+    const float decay = ev[n_valid - 1];
+    for (int r = 0; r < d16 / 16; ++r) {
+      float* sp = Ss + (r * 16 + lq * 4) * VROW + wave * 16 + lr;
+      f32x4 acc = {sp[0] * decay, sp[VROW] * decay, sp[2 * VROW] * decay, sp[3 * VROW] * decay};
+      const float* ka = Ks + lq * QROW + r * 16 + lr;
+      const float* vb = Vs + lq * VROW + wave * 16 + lr;
+      for (int s0 = 0; s0 < L; s0 += 4)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[s0 * QROW] * cv[s0 + lq], vb[s0 * VROW], acc, 0, 0, 0);
+      sp[0] = acc[0];
+      sp[VROW] = acc[1];
+      sp[2 * VROW] = acc[2];
+      sp[3 * VROW] = acc[3];
+    }
+    for (int k = tid; k < d16; k += ML_THREADS) {
+      float a = nv[k] * decay;
+      for (int s_ = 0; s_ < n_valid; ++s_) a = fmaf(cv[s_], Ks[s_ * QROW + k], a);
+      nv[k] = a;
+    }
+    m0 = mv[n_valid - 1];
+  }
+  __syncthreads();
+  for (int i = tid; i < d * DVS; i += ML_THREADS) {
+    const int k = i / DVS, c = i % DVS;
+    if (col0 + c < dv) st[(size_t)k * dv + col0 + c] = Ss[k * VROW + c];
+  }
+  if (slice == 0) {
+    float* o = nm + ((size_t)b * H + h) * (d + 1);
+    for (int k = tid; k < d; k += ML_THREADS) o[k] = nv[k];
+    if (tid == 0) o[d] = m0;
+  }
+}
+
+// out[t, head] = raw / rms(raw) * w * sigmoid(g) (a wave a token and head); the workgroup of a sequence's last token
+// puts the head's n and m into the state; a padding row gets zeros.
+template <typename T>
+__global__ __launch_bounds__(WAVE) void mlstm_finish_kernel(const float* __restrict__ raw, const float* __restrict__ proj,
+                                                            const float* __restrict__ w_norm, const float* __restrict__ nm,
+                                                            float* __restrict__ state, const int* __restrict__ cu_seqlens,
+                                                            const int* __restrict__ seq_slot, T* __restrict__ out, int B,
+                                                            int H, int d, int dv, float eps, int n_slots) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  int lo = 0, hi = B - 1;                         // the sequence of token t
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (cu_seqlens[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  const int b = lo, slot = seq_slot[b];
+  T* o = out + (size_t)t * H * dv + h * dv;
+  if (slot < 0 || slot >= n_slots) {
+    for (int c = lane; c < dv; c += WAVE) o[c] = from_f32<T>(0.f);
+    return;
+  }
+  const float* r = raw + (size_t)t * H * dv + h * dv;
+  float sq = 0.f;
+  for (int c = lane; c < dv; c += WAVE) sq = fmaf(r[c], r[c], sq);
+  sq = wave_sum(sq);
+  const float rsq = 1.0f / sqrtf(sq / (float)dv + eps);
+  const float* g = proj + (size_t)t * (2 * H * d + 2 * H * dv + 2 * H) + 2 * H * d + H * dv + h * dv;
+  for (int c = lane; c < dv; c += WAVE) o[c] = from_f32<T>(r[c] * rsq * w_norm[h * dv + c] / (1.0f + expf(-g[c])));
+  if (t == cu_seqlens[b + 1] - 1) {
+    const float* src = nm + ((size_t)b * H + h) * (d + 1);
+    float* dst = state + ((size_t)slot * H + h) * ((size_t)d * dv + d + 1) + (size_t)d * dv;
+    for (int k = lane; k <= d; k += WAVE) dst[k] = src[k];
+  }
+}
+
+LdsAllowance ml_allow_chunk64, ml_allow_chunk16;
 }  // namespace
+
+// The recurrence a chunk at a time (see mlstm_chunk_kernel).  chunk: 64 (steps of whole prompts) or 16 (single tokens).
+// raw: float32 [T, H dv] and nm: float32 [B, H (d + 1)], scratch of the caller.  Returns YALM_ERR_ARG where the sizes
+// do not fit its LDS (yalm_mlstm_scan then serves).  T: the step's tokens, the last sequence's last token being T - 1.
+extern "C" int yalm_mlstm_chunks(const float* proj, const float* b_i, const float* b_f, const float* w_norm, float* state,
+                                 float* raw, float* nm, const int* cu_seqlens, const int* seq_slot, void* out, int T,
+                                 int B, int H, int d, int dv, float q_scale, float cap, float floor_, float eps,
+                                 int n_slots, int chunk, int dtype, hipStream_t stream) {
+  if (B <= 0 || T <= 0) return YALM_OK;
+  if (H <= 0 || d <= 0 || dv <= 0 || n_slots <= 0 || cap < 0.f || H > 65535 || B > 65535 ||
+      (chunk != 64 && chunk != 16) || (dtype != YALM_F32 && dtype != YALM_BF16))
+    return YALM_ERR_ARG;
+  const int d16 = (d + 15) / 16 * 16;
+  const size_t lds = (chunk == 64 ? chunk_lds_floats<64>(d16) : chunk_lds_floats<16>(d16)) * sizeof(float);
+  if (lds > 150 * 1024) return YALM_ERR_ARG;
+  dim3 grid(ceil_div(dv, DVS), H, B);
+  if (chunk == 64) {
+    auto kernel = &mlstm_chunk_kernel<64>;
+    if (lds > 64 * 1024)
+      if (int rc = allow_dynamic_lds(ml_allow_chunk64, (const void*)kernel, 150 * 1024); rc != YALM_OK) return rc;
+    kernel<<<grid, ML_THREADS, lds, stream>>>(proj, b_i, b_f, state, nm, cu_seqlens, seq_slot, raw, H, d, dv, q_scale, cap,
+                                              floor_, n_slots);
+  } else {
+    auto kernel = &mlstm_chunk_kernel<16>;
+    if (lds > 64 * 1024)
+      if (int rc = allow_dynamic_lds(ml_allow_chunk16, (const void*)kernel, 150 * 1024); rc != YALM_OK) return rc;
+    kernel<<<grid, ML_THREADS, lds, stream>>>(proj, b_i, b_f, state, nm, cu_seqlens, seq_slot, raw, H, d, dv, q_scale, cap,
+                                              floor_, n_slots);
+  }
+  if (int rc = launch_status(); rc != YALM_OK) return rc;
+  if (dtype == YALM_F32)
+    mlstm_finish_kernel<float><<<dim3(T, H), WAVE, 0, stream>>>(raw, proj, w_norm, nm, state, cu_seqlens, seq_slot, (float*)out,
+                                                                B, H, d, dv, eps, n_slots);
+  else
+    mlstm_finish_kernel<bf16><<<dim3(T, H), WAVE, 0, stream>>>(raw, proj, w_norm, nm, state, cu_seqlens, seq_slot, (bf16*)out, B,
+                                                               H, d, dv, eps, n_slots);
+  return launch_status();
+}
+
+// the LDS bytes yalm_mlstm_chunks needs for key heads of d with chunks of `chunk` tokens
+extern "C" long yalm_mlstm_chunks_lds(int d, int chunk) {
+  const int d16 = (d + 15) / 16 * 16;
+  return (long)((chunk == 64 ? chunk_lds_floats<64>(d16) : chunk_lds_floats<16>(d16)) * sizeof(float));
+}
 
 // proj float32 [T, 2 H d + 2 H dv + 2 H]; state float32 [n_slots, H, d dv + d + 1]; out `dtype` [T, H dv];
 // cu_seqlens int32 [B + 1] (the tokens of sequence b are rows cu_seqlens[b] .. cu_seqlens[b + 1] - 1, in order),

@@ -13,9 +13,9 @@
 #include "yalm_hip.h"
 
 namespace {
-constexpr int PACK_THREADS = 256;
-
-template <typename T>
+// a row of a few hundred numbers takes 256 threads, a real model's thousands 1,024 (a decode step has few tokens, and a
+// thread's loads wait for each other's results in turn: the fewer rounds the better)
+template <typename T, int PACK_THREADS>
 __global__ __launch_bounds__(PACK_THREADS) void qkv_pack_kernel(
     const float* __restrict__ qkv, const float* __restrict__ bias, const float* __restrict__ w_q,
     const float* __restrict__ w_k, float eps, float temp_coef, int temp_every, float q_scale, float* __restrict__ v_first,
@@ -30,6 +30,7 @@ __global__ __launch_bounds__(PACK_THREADS) void qkv_pack_kernel(
   const int Q = n_heads * d, K = n_kv_heads * d, V = n_kv_heads * dv, N = Q + K + V;
   const float* src = qkv + (size_t)t * N;
   float sq = 0.f, sk = 0.f;
+#pragma unroll 4
   for (int i = tid; i < N; i += PACK_THREADS) {
     const float v = src[i] + (bias != nullptr ? bias[i] : 0.f);
     row[i] = v;
@@ -109,14 +110,22 @@ extern "C" int yalm_qkv_pack(const float* qkv, const float* bias, const float* w
     return YALM_ERR_ARG;
   const size_t lds = (size_t)(n_heads * d + n_kv_heads * (d + dv)) * sizeof(float);
   if (lds > 64 * 1024) return YALM_ERR_ARG;
+  const bool wide = n_heads * d + n_kv_heads * (d + dv) >= 2048;
 #define YALM_PACK(TYPE)                                                                                              \
-  qkv_pack_kernel<TYPE><<<T, PACK_THREADS, lds, stream>>>(                                                           \
+  if (wide) YALM_PACK_N(TYPE, 1024); else YALM_PACK_N(TYPE, 256)
+#define YALM_PACK_N(TYPE, NT)                                                                                        \
+  qkv_pack_kernel<TYPE, NT><<<T, NT, lds, stream>>>(                                                                 \
       qkv, bias, w_q, w_k, eps, temp_coef, temp_every, q_scale, v_first, blend, lam, (TYPE*)q_out, (TYPE*)k_stage,    \
       (TYPE*)v_stage, seq_tile0, (TYPE*)k_pages, (TYPE*)v_pages, block_table, table_stride, ring_pages, tok_seq,     \
       tok_pos, seq_slot, seq_len, n_heads, n_kv_heads, d, dv, pad, n_pages, page_layout)
-  if (dtype == YALM_F32) YALM_PACK(float);
-  else if (dtype == YALM_BF16) YALM_PACK(bf16);
-  else return YALM_ERR_DTYPE;
+  if (dtype == YALM_F32) {
+    YALM_PACK(float);
+  } else if (dtype == YALM_BF16) {
+    YALM_PACK(bf16);
+  } else {
+    return YALM_ERR_DTYPE;
+  }
 #undef YALM_PACK
+#undef YALM_PACK_N
   return launch_status();
 }

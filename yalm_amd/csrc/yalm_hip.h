@@ -330,6 +330,16 @@ int yalm_mlstm_scan(const float* proj, const float* b_i, const float* b_f, const
                     const int* cu_seqlens, const int* seq_slot, void* out, int B, int H, int d, int dv, float q_scale,
                     float cap, float floor_, float eps, int n_slots, int dtype, hipStream_t stream);
 
+// The same recurrence a chunk of tokens at a time on the matrix cores, in float32 (chunk 64: steps of whole prompts,
+// 16: single tokens); a workgroup owns 64 columns of a (sequence, head).  raw float32 [T, H dv] and nm float32
+// [B, H (d + 1)]: scratch of the caller.  T: rows of proj and out.  YALM_ERR_ARG where yalm_mlstm_chunks_lds(d, chunk)
+// exceeds 150 KB.
+int yalm_mlstm_chunks(const float* proj, const float* b_i, const float* b_f, const float* w_norm, float* state, float* raw,
+                      float* nm, const int* cu_seqlens, const int* seq_slot, void* out, int T, int B, int H, int d, int dv,
+                      float q_scale, float cap, float floor_, float eps, int n_slots, int chunk, int dtype,
+                      hipStream_t stream);
+long yalm_mlstm_chunks_lds(int d, int chunk);
+
 // Yardsticks for the measurement (probes.hip): a kernel that only reads `bytes` bytes once with `workgroups`
 // workgroups (out: 1,024 words of scratch), and a loop of matrix-core instructions on registers (shape 32:
 // v_mfma_f32_32x32x16_bf16, 16: v_mfma_f32_16x16x32_bf16; *flops, host memory, receives the launch's operations).

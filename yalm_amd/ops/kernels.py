@@ -896,6 +896,36 @@ def mlstm_fits(d, dv):
     return 0 < dv <= MLSTM_MAX_VDIM and d > 0 and (d * dv + 3 * d + dv + groups * dv) * 4 <= MLSTM_MAX_LDS
 
 
+def mlstm_chunk(d, prompt):
+    """The chunk with which mlstm_chunks takes key heads of d: 64 tokens for steps of whole prompts where that fits its
+    LDS, else 16; 0 if not even that fits (mlstm_scan then serves)."""
+    for chunk in ((64, 16) if prompt else (16,)):
+        if library.lib().yalm_mlstm_chunks_lds(int(d), chunk) <= MLSTM_MAX_LDS:
+            return chunk
+    return 0
+
+
+def mlstm_chunks(proj, b_i, b_f, w_norm, state, raw, nm, cu_seqlens, seq_slot, out, n_heads, d, dv, q_scale, cap, floor, eps,
+                 chunk):
+    """mlstm_scan's result a chunk of `chunk` tokens at a time on the matrix cores, in float32 arithmetic (the same
+    recurrence written over a chunk: scores q . k weighted by the gates inside it, the state carried between chunks).
+    raw float32 [T, H dv] and nm float32 [B, H (d + 1)] are scratch."""
+    T = proj.shape[0]
+    B = seq_slot.shape[0]
+    H = n_heads
+    if chunk not in (16, 64) or library.lib().yalm_mlstm_chunks_lds(int(d), chunk) > MLSTM_MAX_LDS:
+        raise ValueError("mlstm_chunks: key heads of %d do not fit chunks of %r" % (d, chunk))
+    n_slots = state.shape[0]
+    library.check(library.lib().yalm_mlstm_chunks(
+        _need(proj, "proj", torch.float32, (T, 2 * H * d + 2 * H * dv + 2 * H)), _need(b_i, "b_i", torch.float32, (H,)),
+        _need(b_f, "b_f", torch.float32, (H,)), _need(w_norm, "w_norm", torch.float32, (H * dv,)),
+        _need(state, "state", torch.float32, (n_slots, H * (d * dv + d + 1))), _need(raw, "raw", torch.float32, (T, H * dv)),
+        _need(nm, "nm", torch.float32, (B, H * (d + 1))), _need(cu_seqlens, "cu_seqlens", torch.int32, (B + 1,)),
+        _need(seq_slot, "seq_slot", torch.int32, (B,)), _need(out, "out", None, (T, H * dv)), T, B, H, d, dv, float(q_scale),
+        float(cap), float(floor), float(eps), n_slots, int(chunk), dtype_code(out.dtype), _stream()), "mlstm_chunks")
+    return out
+
+
 def mlstm_scan(proj, b_i, b_f, w_norm, state, cu_seqlens, seq_slot, out, n_heads, d, dv, q_scale, cap, floor, eps):
     """The matrix-memory recurrence over the tokens of a step.  proj float32 [T, 2 H d + 2 H dv + 2 H] = q | k | v | g |
     z_i | z_f; with i = cap tanh((z_i + b_i) / cap), f = logsigmoid(cap tanh((z_f + b_f) / cap)) (cap 0: uncapped):

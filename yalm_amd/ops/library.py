@@ -65,12 +65,14 @@ _SIGNATURES = {
     "yalm_embed_sinusoid": (_I, [_P, _I, _P, _P, _P, _F, _P, _I, _I, _I, _P]),
     "yalm_qkv_pack": (_I, [_P, _P, _P, _P, _F, _F, _I, _F, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P,
                            _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_mlstm_chunks": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _F, _F, _I, _I, _I, _P]),
+    "yalm_mlstm_chunks_lds": (ctypes.c_long, [_I, _I]),
     "yalm_mlstm_scan": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _F, _F, _I, _I, _P]),
     "yalm_probe_read": (_I, [_P, ctypes.c_long, _P, _I, _P]),
     "yalm_probe_mfma": (_I, [_I, _I, _I, _P, _P, _P]),
 }
 
-ABI_VERSION = 29
+ABI_VERSION = 30
 
 
 class KernelError(RuntimeError):

@@ -44,7 +44,8 @@ class PreNormResidualBlock(Part):
 class ParallelResidualBlock(Part):
     """x += mixer(h) + feed_forward(h) with h = norm(x): one norm, and both sublayers read its output.  Members: norm,
     mixer, and optionally feed_forward.  Each sublayer adds its result to the float32 stream in the epilogue of its
-    last product, the mixer first."""
+    last product, the mixer first.  In a decode step the layer ends with the norm that reads the stream next (the next
+    layer's, or the final one, whose output the head's product then takes as it is)."""
 
     def __init__(self, layer_spec, dim, prefix=""):
         super().__init__(None, dim, layer_spec.prefix)
@@ -71,6 +72,11 @@ class ParallelResidualBlock(Part):
         self.mixer.forward(h, x, ctx, line, writes_cache)
         if self.feed_forward is not None:
             self.feed_forward.forward(h, x, ctx)
+        if ctx.mode == "decode" and next_norm is not None and hasattr(next_norm, "fused"):
+            other = "block.h" if h.data_ptr() != ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype).data_ptr() else "block.h2"
+            ahead = ctx.ws.get(other, (x.shape[0], self.dim), ctx.act_dtype)      # not the buffer this layer has just read
+            next_norm.forward(x, ahead, ctx)
+            ctx.normed[id(next_norm)] = (ahead, None, None)
 
 
 class StreamInput:

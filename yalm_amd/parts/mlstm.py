@@ -6,7 +6,9 @@ Per token and head: q = W_q h * q_scale, k = W_k h, v = W_v h; i = cap tanh((W_i
 f = logsigmoid(cap tanh((W_f h + b_f) / cap)); m' = max(f + m, i); S' = exp(f + m - m') S + exp(i - m') k v^T;
 n' likewise with k; o = S'^T q / (max(|n' . q|, exp(-m')) + floor).  Each head's o is divided by its root mean
 square, the heads side by side are multiplied by a weight and by sigmoid(W_g h), and W_o adds the result to the
-residual stream.  The six projections are one matrix; everything behind it is float32 in one kernel."""
+residual stream.  The six projections are one matrix; everything behind it is float32: the recurrence a chunk of
+tokens at a time on the matrix cores (64 tokens in a step of whole prompts, 16 around a single token), the heads'
+norm and gate in a second kernel; key heads too wide for that take the kernel that walks token by token."""
 import torch
 
 from ..cache.manager import StateRequest
@@ -30,9 +32,9 @@ class MLSTM(Part):
         self.q_scale = float(p.get("q_scale") or self.key_dim ** -0.5)
         self.floor = float(p.get("floor", 1e-6))
         self.eps = float(p.get("eps", 1e-6))
-        if not kernels.mlstm_fits(self.key_dim, self.value_dim):
-            raise ValueError("mLSTM heads of %d x %d are not offered (values up to %d a head, the state within %d KB)"
-                             % (self.key_dim, self.value_dim, kernels.MLSTM_MAX_VDIM, kernels.MLSTM_MAX_LDS // 1024))
+        if not kernels.mlstm_fits(self.key_dim, self.value_dim) and not kernels.mlstm_chunk(self.key_dim, False):
+            raise ValueError("mLSTM heads of %d x %d are not offered: neither 64 columns of the state nor the whole of it "
+                             "fit %d KB" % (self.key_dim, self.value_dim, kernels.MLSTM_MAX_LDS // 1024))
         self.names = dict(NAMES)
         self.names.update(p.get("tensors") or {})
         self.qk, self.vv = self.n_heads * self.key_dim, self.n_heads * self.value_dim
@@ -70,7 +72,8 @@ class MLSTM(Part):
         return 2 * self.qk + 2 * self.vv + 2 * self.n_heads
 
     def describe(self, compute_dtype):
-        return "mLSTM, %d heads of %d x %d: one token after another, float32" % (self.n_heads, self.key_dim, self.value_dim), False
+        how = "chunks on the matrix cores in float32" if kernels.mlstm_chunk(self.key_dim, True) else "one token after another, float32"
+        return "mLSTM, %d heads of %d x %d: %s" % (self.n_heads, self.key_dim, self.value_dim, how), False
 
     def forward(self, h, x, ctx, line, writes_cache=True):
         T = h.shape[0]
@@ -78,6 +81,14 @@ class MLSTM(Part):
         self._gemm(ctx, h, self.w_in, proj, kernels.EPI_STORE_F32)
         o = ctx.ws.get("mlstm.o", (T, self.vv), h.dtype)
         state = ctx.cache.group_of(line).line_state(line)
-        kernels.mlstm_scan(proj, self.b_i, self.b_f, self.w_norm, state, ctx.cu_seqlens, ctx.seq_slot, o, self.n_heads,
-                           self.key_dim, self.value_dim, self.q_scale, self.gate_cap, self.floor, self.eps)
+        chunk = kernels.mlstm_chunk(self.key_dim, ctx.mode == "prefill")
+        if chunk:
+            raw = ctx.ws.get("mlstm.raw", (T, self.vv), torch.float32)
+            nm = ctx.ws.get("mlstm.nm", (ctx.seq_slot.shape[0], self.n_heads * (self.key_dim + 1)), torch.float32)
+            kernels.mlstm_chunks(proj, self.b_i, self.b_f, self.w_norm, state, raw, nm, ctx.cu_seqlens, ctx.seq_slot, o,
+                                 self.n_heads, self.key_dim, self.value_dim, self.q_scale, self.gate_cap, self.floor, self.eps,
+                                 chunk)
+        else:
+            kernels.mlstm_scan(proj, self.b_i, self.b_f, self.w_norm, state, ctx.cu_seqlens, ctx.seq_slot, o, self.n_heads,
+                               self.key_dim, self.value_dim, self.q_scale, self.gate_cap, self.floor, self.eps)
         self._gemm(ctx, o, self.wo, x, kernels.EPI_ADD_F32)
