@@ -172,7 +172,7 @@ class GedunexConfig:
                 if m.get("v_mix"):
                     blend = "later" if blend_seen else "first"
                     blend_seen = True
-                position = PartSpec("distance_slopes", {"n_heads": m["heads"], "exponent": SLOPE_EXPONENT, "window": window})
+                position = PartSpec("distance_slopes", {"n_heads": m["heads"], "exponent": SLOPE_EXPONENT})
                 qt = m.get("q_temp")
                 mixer = PartSpec("shaped_attention", {
                     "n_heads": m["heads"], "n_kv_heads": m["kv_heads"], "key_dim": m["dim"], "value_dim": m["vdim"],

@@ -28,8 +28,11 @@ struct ScoreBias {
   int n;
   float softcap;               // score <- softcap tanh(score / softcap) before the distance's term (0: no cap)
   const float* sink_logit;     // [heads]: a logit in the softmax's denominator that has no key and no value (null: none)
+  const float* slope;          // [heads]: -slope[head] * distance is added to every score (null: none)
   __device__ __forceinline__ float at(int head, int distance) const {
-    return table != nullptr ? table[(size_t)head * n + min(max(distance, 0), n - 1)] : 0.f;
+    float term = table != nullptr ? table[(size_t)head * n + min(max(distance, 0), n - 1)] : 0.f;
+    if (slope != nullptr) term -= slope[head] * (float)distance;
+    return term;
   }
   // the score of a scaled product at a distance
   __device__ __forceinline__ float shaped(float s, int head, int distance) const {
@@ -334,12 +337,12 @@ extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const v
                                  const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads,
                                  int n_kv_heads, int head_dim, int window, int dtype, int force_simple,
                                  const float* score_bias, int n_bias, float softcap, const float* sink_logit,
-                                 hipStream_t stream) {
+                                 const float* slopes, hipStream_t stream) {
   if (T <= 0) return YALM_OK;
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_tiles <= 0) return YALM_ERR_ARG;
   if ((score_bias != nullptr && n_bias <= 0) || softcap < 0.f) return YALM_ERR_ARG;
-  const ScoreBias sb = {score_bias, n_bias, softcap, sink_logit};
-  const ScoreShape shape = {score_bias, n_bias, softcap, sink_logit};
+  const ScoreBias sb = {score_bias, n_bias, softcap, sink_logit, slopes};
+  const ScoreShape shape = {score_bias, n_bias, softcap, sink_logit, slopes};
   dim3 grid(T, n_heads);
   if (dtype == YALM_F32) {
     if (head_dim <= ACC_SMALL * WAVE)
@@ -376,7 +379,7 @@ extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void*
                                  hipStream_t stream) {
   return yalm_attn_prefill_lse(q, k_stage, v_stage, out, nullptr, nullptr, cu_seqlens, seq_tile0, tok_seq, tok_pos, tile_order,
                                n_order, T, B, n_tiles, n_heads, n_kv_heads, head_dim, window, dtype, force_simple,
-                               nullptr, 0, 0.f, nullptr, stream);
+                               nullptr, 0, 0.f, nullptr, nullptr, stream);
 }
 
 // merges the partial results of the splits (also used by the MFMA kernel)
@@ -403,12 +406,12 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
                     int B, int n_heads, int n_kv_heads, int head_dim, int window, int n_splits, int n_pages,
                     int page_layout, int dtype, int force_simple, const SinkArgs& sinks, const int* step_max_len,
                     const int* seq_order, const float* score_bias, int n_bias, float softcap,
-                    const float* sink_logit, hipStream_t stream) {
+                    const float* sink_logit, const float* slopes, hipStream_t stream) {
   if (B <= 0) return YALM_OK;
-  const ScoreShape shape = {score_bias, n_bias, softcap, sink_logit};
+  const ScoreShape shape = {score_bias, n_bias, softcap, sink_logit, slopes};
   if ((score_bias != nullptr && n_bias <= 0) || softcap < 0.f || (shape.any() && sinks.n_sinks > 0))
     return YALM_ERR_ARG;                                                // kept first positions are scored unshaped
-  const ScoreBias sb = {score_bias, n_bias, softcap, sink_logit};
+  const ScoreBias sb = {score_bias, n_bias, softcap, sink_logit, slopes};
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_splits <= 0 || ring_pages <= 0 ||
       !page_layout_ok(page_layout, head_dim))
     return YALM_ERR_ARG;
@@ -459,11 +462,11 @@ extern "C" int yalm_attn_decode_lse(const void* q, const void* k_pages, const vo
                                     int head_dim, int window, int n_splits, int n_pages, int page_layout, int dtype,
                                     int force_simple, const int* step_max_len, const int* seq_order,
                                     const float* score_bias, int n_bias, float softcap, const float* sink_logit,
-                                    hipStream_t stream) {
+                                    const float* slopes, hipStream_t stream) {
   SinkArgs none = {};
   return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, lse,
                          partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, dtype,
-                         force_simple, none, step_max_len, seq_order, score_bias, n_bias, softcap, sink_logit, stream);
+                         force_simple, none, step_max_len, seq_order, score_bias, n_bias, softcap, sink_logit, slopes, stream);
 }
 
 extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -472,7 +475,7 @@ extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* 
                                 int n_splits, int n_pages, int dtype, int force_simple, hipStream_t stream) {
   return yalm_attn_decode_lse(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out,
                               nullptr, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages,
-                              YALM_PAGE_ROWS, dtype, force_simple, nullptr, nullptr, nullptr, 0, 0.f, nullptr, stream);
+                              YALM_PAGE_ROWS, dtype, force_simple, nullptr, nullptr, nullptr, 0, 0.f, nullptr, nullptr, stream);
 }
 
 extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -508,7 +511,7 @@ extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const 
   sk.n_sinks = n_sinks;
   return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, nullptr,
                          partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, dtype,
-                         force_simple, sk, step_max_len, seq_order, nullptr, 0, 0.f, nullptr, stream);
+                         force_simple, sk, step_max_len, seq_order, nullptr, 0, 0.f, nullptr, nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------

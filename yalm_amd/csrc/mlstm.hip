@@ -132,6 +132,15 @@ constexpr int DVS = 64;                           // columns of S a workgroup ow
 constexpr int VROW = DVS + 16;                    // LDS row strides (floats)
 constexpr float NEVER = -3.0e38f;
 
+// A barrier that waits for the wave's LDS traffic only.  __syncthreads() carries a fence that also waits for every global
+// load in flight, and the next chunk's operands are meant to stay in flight across the barriers of this chunk's work.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0x3F | (0x7 << 4) | (0x0 << 8) | (0x3 << 14));      // lgkmcnt(0), nothing else
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 template <int L>
 __host__ __device__ constexpr size_t chunk_lds_floats(int d16) {
   return (size_t)d16 * VROW + 2 * (size_t)L * (d16 + 4) + (size_t)L * VROW + (size_t)L * (L + 4) + d16 + 8 * L;
@@ -168,35 +177,73 @@ __global__ __launch_bounds__(ML_THREADS) void mlstm_chunk_kernel(
   const int per = d * dv + d + 1;
   float* st = state + ((size_t)slot * H + h) * per;
   const int col0 = slice * DVS;
-  for (int i = tid; i < d16 * DVS; i += ML_THREADS) {
-    const int k = i / DVS, c = i % DVS;
-    Ss[k * VROW + c] = k < d && col0 + c < dv ? st[(size_t)k * dv + col0 + c] : 0.f;
+  // a wave takes rows wave, wave + 4, ... of the 64 columns, eight rows' loads in flight at a time
+  for (int kb = wave; kb < d16; kb += 32) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = kb + 4 * j;
+      v[j] = k < d && col0 + lane < dv ? st[(size_t)k * dv + col0 + lane] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (kb + 4 * j < d16) Ss[(kb + 4 * j) * VROW + lane] = v[j];
   }
   for (int k = tid; k < d16; k += ML_THREADS) nv[k] = k < d ? st[(size_t)d * dv + k] : 0.f;
   float m0 = st[(size_t)d * dv + d];
   const int N = 2 * H * d + 2 * H * dv + 2 * H;
   constexpr int RT = L / 16;                      // row tiles of a chunk
 
+  // A chunk's queries, keys, values and gate inputs are asked for a chunk ahead and wait in registers while the
+  // chunk before is worked (a workgroup has its compute unit alone: nobody else would hide the loads' latency).
+  // Thread (wave, lane) holds tokens wave, wave + 4, ... and elements lane, lane + 64, ...
+  constexpr int TJ = L / 4, KJ = L == 64 ? 2 : 5; // d16 <= 64 KJ where the LDS fits
+  float qreg[TJ][KJ], kreg[TJ][KJ], vreg[TJ], zreg[2] = {0.f, 0.f};
+  auto fetch = [&](int t0) {
+    const int n_valid = min(L, t_end - t0);
+#pragma unroll
+    for (int jt = 0; jt < TJ; ++jt) {
+      const int t = wave + 4 * jt;
+      vreg[jt] = t < n_valid && col0 + lane < dv ? proj[(size_t)(t0 + t) * N + 2 * H * d + h * dv + col0 + lane] : 0.f;
+#pragma unroll
+      for (int jk = 0; jk < KJ; ++jk) {
+        const int k = lane + WAVE * jk;
+        const bool ok = t < n_valid && k < d;
+        const float* row = proj + (size_t)(t0 + (ok ? t : 0)) * N + h * d + (ok ? k : 0);
+        qreg[jt][jk] = ok ? row[0] : 0.f;
+        kreg[jt][jk] = ok ? row[H * d] : 0.f;
+      }
+    }
+    if (wave == 0 && lane < n_valid) {
+      const float* row = proj + (size_t)(t0 + lane) * N + 2 * H * d + 2 * H * dv;
+      zreg[0] = row[h];
+      zreg[1] = row[H + h];
+    }
+  };
+  fetch(t_begin);
+  const float bias_i = b_i[h], bias_f = b_f[h];
+
   for (int t0 = t_begin; t0 < t_end; t0 += L) {
     const int n_valid = min(L, t_end - t0);
     __syncthreads();                              // the chunk before is done with Qs, Ks, Vs, Ps and the vectors
-    for (int i = tid; i < L * d16; i += ML_THREADS) {
-      const int t = i / d16, k = i % d16;
-      const bool ok = t < n_valid && k < d;
-      const float* row = proj + (size_t)(t0 + t) * N;
-      Qs[t * QROW + k] = ok ? row[h * d + k] * q_scale : 0.f;
-      Ks[t * QROW + k] = ok ? row[H * d + h * d + k] : 0.f;
-    }
-    for (int i = tid; i < L * DVS; i += ML_THREADS) {
-      const int t = i / DVS, c = i % DVS;
-      Vs[t * VROW + c] = t < n_valid && col0 + c < dv ? proj[(size_t)(t0 + t) * N + 2 * H * d + h * dv + col0 + c] : 0.f;
+#pragma unroll
+    for (int jt = 0; jt < TJ; ++jt) {
+      const int t = wave + 4 * jt;
+      Vs[t * VROW + lane] = vreg[jt];
+#pragma unroll
+      for (int jk = 0; jk < KJ; ++jk) {
+        const int k = lane + WAVE * jk;
+        if (k < d16) {
+          Qs[t * QROW + k] = qreg[jt][jk] * q_scale;
+          Ks[t * QROW + k] = kreg[jt][jk];
+        }
+      }
     }
     if (wave == 0) {                              // the gates of the chunk: sums and maxima along it, a lane a token
       float f = 0.f, zi = NEVER;
       if (lane < n_valid) {
-        const float* row = proj + (size_t)(t0 + lane) * N + 2 * H * d + 2 * H * dv;
-        zi = row[h] + b_i[h];
-        float zf = row[H + h] + b_f[h];
+        zi = zreg[0] + bias_i;
+        float zf = zreg[1] + bias_f;
         if (cap > 0.f) {
           zi = cap * tanhf(zi / cap);
           zf = cap * tanhf(zf / cap);
@@ -228,87 +275,130 @@ __global__ __launch_bounds__(ML_THREADS) void mlstm_chunk_kernel(
       }
     }
     __syncthreads();
+    if (t0 + L < t_end) fetch(t0 + L);             // the next chunk's loads fly while this one is worked
+    if (tid < 4 * L) {                             // q_t . n0: four threads a token, a quarter of the elements each
+      const int t = tid / 4, part = tid % 4;
+      float a = 0.f;
+      for (int k = part; k < d16; k += 4) a = fmaf(Qs[t * QROW + k], nv[k], a);
+      a += __shfl_xor(a, 1, WAVE);
+      a += __shfl_xor(a, 2, WAVE);
+      if (part == 0) qn[t] = a;
+    }
     // scores: P[t][s] = (q_t . k_s) exp(w_s - g_t) for s <= t; a wave a tile of 16 tokens
     if (wave < RT) {
+      // the key tiles up to the diagonal side by side: independent sums keep the matrix cores busy, and a query
+      // element is read once for all of them
+      f32x4 acc[RT];
+#pragma unroll
+      for (int c = 0; c < RT; ++c) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      const float* qa = Qs + (wave * 16 + lr) * QROW + lq;
+      const float* kb = Ks + lr * QROW + lq;
+#pragma unroll 4
+      for (int k0 = 0; k0 < d16; k0 += 4) {
+        const float a = qa[k0];
+#pragma unroll
+        for (int c = 0; c < RT; ++c)
+          if (c <= wave) acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, kb[c * 16 * QROW + k0], acc[c], 0, 0, 0);
+      }
+      float sum[4] = {0.f, 0.f, 0.f, 0.f};        // of the rows lq * 4 + v over this lane's columns
+#pragma unroll
       for (int c = 0; c < RT; ++c) {
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        if (c <= wave) {
-          const float* qa = Qs + (wave * 16 + lr) * QROW + lq;
-          const float* kb = Ks + (c * 16 + lr) * QROW + lq;
-          for (int k0 = 0; k0 < d16; k0 += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[k0], kb[k0], acc, 0, 0, 0);
-        }
         const int s_ = c * 16 + lr;
         const float ws = wv[s_];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           const int t = wave * 16 + lq * 4 + v;
-          Ps[t * PROW + s_] = s_ <= t ? acc[v] * expf(ws - gv[t]) : 0.f;
+          const float pv = s_ <= t ? acc[c][v] * expf(ws - gv[t]) : 0.f;
+          Ps[t * PROW + s_] = pv;
+          sum[v] += pv;
         }
       }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) sum[v] += __shfl_xor(sum[v], o, WAVE);
+        if (lr == 0) rs[wave * 16 + lq * 4 + v] = sum[v];
+      }
     }
-    __syncthreads();
-    if (tid < L) {
-      float a = 0.f;
-      for (int s_ = 0; s_ <= tid; ++s_) a += Ps[tid * PROW + s_];
-      rs[tid] = a;
-    } else if (tid >= WAVE && tid < WAVE + L) {
-      const int t = tid - WAVE;
-      float a = 0.f;
-      for (int k = 0; k < d16; ++k) a = fmaf(Qs[t * QROW + k], nv[k], a);
-      qn[t] = a;
-    }
-    __syncthreads();
+    lds_barrier();
     // the tokens' results: P V + exp(m0 - g_t) Q S0, over the denominator
     if (wave < RT) {
-      for (int c = 0; c < DVS / 16; ++c) {
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
-        const float* pa = Ps + (wave * 16 + lr) * PROW + lq;
-        const float* vb = Vs + lq * VROW + c * 16 + lr;
-        for (int s0 = 0; s0 < (wave + 1) * 16; s0 += 4)
-          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[s0], vb[s0 * VROW], acc, 0, 0, 0);
-        const float* qa = Qs + (wave * 16 + lr) * QROW + lq;
-        const float* sb = Ss + lq * VROW + c * 16 + lr;
-        for (int k0 = 0; k0 < d16; k0 += 4)
-          acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[k0], sb[k0 * VROW], acc2, 0, 0, 0);
-        const int col = col0 + c * 16 + lr;
+      constexpr int CT = DVS / 16;                // the four column tiles side by side
+      f32x4 acc[CT], acc2[CT];
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          const int t = wave * 16 + lq * 4 + v;
-          if (t < n_valid && col < dv) {
-            const float e = ev[t];
-            const float den = fmaxf(fabsf(fmaf(e, qn[t], rs[t])), expf(-mv[t])) + floor_;
-            raw[(size_t)(t0 + t) * H * dv + h * dv + col] = fmaf(e, acc2[v], acc[v]) / den;
+      for (int c = 0; c < CT; ++c) acc[c] = acc2[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      const float* pa = Ps + (wave * 16 + lr) * PROW + lq;
+      const float* vb = Vs + lq * VROW + lr;
+#pragma unroll 4
+      for (int s0 = 0; s0 < (wave + 1) * 16; s0 += 4) {
+        const float a = pa[s0];
+#pragma unroll
+        for (int c = 0; c < CT; ++c) acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, vb[s0 * VROW + c * 16], acc[c], 0, 0, 0);
+      }
+      const float* qa = Qs + (wave * 16 + lr) * QROW + lq;
+      const float* sb = Ss + lq * VROW + lr;
+#pragma unroll 4
+      for (int k0 = 0; k0 < d16; k0 += 4) {
+        const float a = qa[k0];
+#pragma unroll
+        for (int c = 0; c < CT; ++c) acc2[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, sb[k0 * VROW + c * 16], acc2[c], 0, 0, 0);
+      }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int t = wave * 16 + lq * 4 + v;
+        if (t < n_valid) {
+          const float e = ev[t];
+          const float inv = 1.0f / (fmaxf(fabsf(fmaf(e, qn[t], rs[t])), expf(-mv[t])) + floor_);
+#pragma unroll
+          for (int c = 0; c < CT; ++c) {
+            const int col = col0 + c * 16 + lr;
+            if (col < dv) raw[(size_t)(t0 + t) * H * dv + h * dv + col] = fmaf(e, acc2[c][v], acc[c][v]) * inv;
           }
         }
       }
     }
-    __syncthreads();
+    lds_barrier();
     // the state behind the chunk: exp(m0 - g_L) S0 + (c K)^T V; wave w owns the column tile w of every row tile
     const float decay = ev[n_valid - 1];
-    for (int r = 0; r < d16 / 16; ++r) {
-      float* sp = Ss + (r * 16 + lq * 4) * VROW + wave * 16 + lr;
-      f32x4 acc = {sp[0] * decay, sp[VROW] * decay, sp[2 * VROW] * decay, sp[3 * VROW] * decay};
-      const float* ka = Ks + lq * QROW + r * 16 + lr;
+    for (int r0 = 0; r0 < d16 / 16; r0 += 4) {    // four row tiles side by side: a value element is read once for them
+      const int nr = min(4, d16 / 16 - r0);
+      float* sp = Ss + (r0 * 16 + lq * 4) * VROW + wave * 16 + lr;
+      f32x4 acc[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float* p = sp + (j < nr ? j : 0) * 16 * VROW;
+        acc[j] = (f32x4){p[0] * decay, p[VROW] * decay, p[2 * VROW] * decay, p[3 * VROW] * decay};
+      }
+      const float* ka = Ks + lq * QROW + r0 * 16 + lr;
       const float* vb = Vs + lq * VROW + wave * 16 + lr;
-      for (int s0 = 0; s0 < L; s0 += 4)
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[s0 * QROW] * cv[s0 + lq], vb[s0 * VROW], acc, 0, 0, 0);
-      sp[0] = acc[0];
-      sp[VROW] = acc[1];
-      sp[2 * VROW] = acc[2];
-      sp[3 * VROW] = acc[3];
+#pragma unroll 4
+      for (int s0 = 0; s0 < L; s0 += 4) {
+        const float bvv = vb[s0 * VROW], cs = cv[s0 + lq];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (j < nr) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[s0 * QROW + j * 16] * cs, bvv, acc[j], 0, 0, 0);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (j < nr) {
+          float* p = sp + j * 16 * VROW;
+          p[0] = acc[j][0];
+          p[VROW] = acc[j][1];
+          p[2 * VROW] = acc[j][2];
+          p[3 * VROW] = acc[j][3];
+        }
     }
     for (int k = tid; k < d16; k += ML_THREADS) {
       float a = nv[k] * decay;
-      for (int s_ = 0; s_ < n_valid; ++s_) a = fmaf(cv[s_], Ks[s_ * QROW + k], a);
+#pragma unroll 8
+      for (int s_ = 0; s_ < L; ++s_) a = fmaf(cv[s_], Ks[s_ * QROW + k], a);      // tokens behind the end weigh 0
       nv[k] = a;
     }
     m0 = mv[n_valid - 1];
   }
   __syncthreads();
-  for (int i = tid; i < d * DVS; i += ML_THREADS) {
-    const int k = i / DVS, c = i % DVS;
-    if (col0 + c < dv) st[(size_t)k * dv + col0 + c] = Ss[k * VROW + c];
-  }
+  if (col0 + lane < dv)
+    for (int k = wave; k < d; k += ML_WAVES) st[(size_t)k * dv + col0 + lane] = Ss[k * VROW + lane];
   if (slice == 0) {
     float* o = nm + ((size_t)b * H + h) * (d + 1);
     for (int k = tid; k < d; k += ML_THREADS) o[k] = nv[k];

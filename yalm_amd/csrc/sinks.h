@@ -15,7 +15,10 @@ struct ScoreShape {
   int n_bias;
   float softcap;
   const float* sink_logit;
-  __host__ __device__ bool any() const { return bias != nullptr || softcap > 0.f || sink_logit != nullptr; }
+  const float* slope;
+  __host__ __device__ bool any() const {
+    return bias != nullptr || softcap > 0.f || sink_logit != nullptr || slope != nullptr;
+  }
 };
 // cap tanh(s / cap) from the exponential instruction (the matrix-core kernels; absolute error about 1e-7 cap)
 __device__ __forceinline__ float soft_cap_fast(float s, float cap) {

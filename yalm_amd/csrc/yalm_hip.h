@@ -168,17 +168,19 @@ long yalm_attn_decode_workspace(int B, int n_heads, int head_dim, int n_splits);
 // softcap (0: none): score <- softcap tanh(score / softcap), after the scaling and before score_bias's term.
 // sink_logit (device, float32 [n_heads]; may be null): a learned logit per head that counts once in the softmax's
 // denominator and has no key and no value (it is not scaled, not capped and gets no distance term; lse counts it).
+// slopes (device, float32 [n_heads]; may be null): -slopes[head] * distance is added to every score, as score_bias's
+// term is, without a table.
 int yalm_attn_prefill_lse(const void* q, const void* k_stage, const void* v_stage, void* out, float* out_f32, float* lse,
                           const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
                           const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads, int n_kv_heads,
                           int head_dim, int window, int dtype, int force_simple, const float* score_bias, int n_bias,
-                          float softcap, const float* sink_logit, hipStream_t stream);
+                          float softcap, const float* sink_logit, const float* slopes, hipStream_t stream);
 int yalm_attn_decode_lse(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                          int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                          float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
                          int n_splits, int n_pages, int page_layout, int dtype, int force_simple,
                          const int* step_max_len, const int* seq_order, const float* score_bias, int n_bias,
-                         float softcap, const float* sink_logit, hipStream_t stream);
+                         float softcap, const float* sink_logit, const float* slopes, hipStream_t stream);
 
 // Attention sinks beside a window (src/infer.cpp:305-319, 486-488): the first n_sinks positions of a
 // sequence stay visible when the window has moved past them, and each then counts as lying

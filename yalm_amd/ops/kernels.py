@@ -580,18 +580,20 @@ def _bias(score_bias, n_heads):
     return _need(score_bias, "score_bias", torch.float32, (n_heads, n)), n
 
 
-def _shape(softcap, sink_logit, n_heads):
-    """(cap, address of the sink logits): softcap > 0 replaces every scaled score s by softcap tanh(s / softcap) before
-    the score bias; sink_logit, float32 [n_heads] on the device, is a logit per head that counts once in the softmax's
-    denominator and has neither key nor value."""
+def _shape(softcap, sink_logit, n_heads, slopes=None):
+    """(cap, address of the sink logits, address of the slopes): softcap > 0 replaces every scaled score s by softcap
+    tanh(s / softcap) before the score bias; sink_logit, float32 [n_heads] on the device, is a logit per head that counts
+    once in the softmax's denominator and has neither key nor value; slopes, float32 [n_heads] on the device, adds
+    -slopes[head] * (query position - key position) to every score (what a score_bias table of slope times distance
+    would add, without the table)."""
     cap = float(softcap or 0.0)
     if cap < 0.0:
         raise ValueError("a score cap must be positive (0: none)")
-    return cap, _opt(sink_logit, "sink_logit", torch.float32, (n_heads,))
+    return cap, _opt(sink_logit, "sink_logit", torch.float32, (n_heads,)), _opt(slopes, "slopes", torch.float32, (n_heads,))
 
 
 def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_pos, n_heads, n_kv_heads, head_dim,
-                 window, tile_order=None, lse=None, out_f32=None, score_bias=None, softcap=0.0, sink_logit=None):
+                 window, tile_order=None, lse=None, out_f32=None, score_bias=None, softcap=0.0, sink_logit=None, slopes=None):
     """Causal (and windowed) attention of packed sequences that start at position 0, over
     the keys and values that rope_kv_write staged for this step.  tile_order (device int32,
     from prefill_tile_order) only changes the order of the work.  lse (float32 [T, n_heads], optional)
@@ -620,7 +622,7 @@ def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_p
     library.check(library.lib().yalm_attn_prefill_lse(p_q, p_k, p_v, p_o, p_o32, p_lse, p_cu, p_t0, p_ts, p_tp, p_or, n_order,
                                                       T, B, n_tiles, n_heads, n_kv_heads, head_dim, int(window),
                                                       dtype_code(dt), 1 if FORCE_SIMPLE else 0,
-                                                      *_bias(score_bias, n_heads), *_shape(softcap, sink_logit, n_heads),
+                                                      *_bias(score_bias, n_heads), *_shape(softcap, sink_logit, n_heads, slopes),
                                                       _stream()),
                   "attn_prefill")
     return out
@@ -632,7 +634,7 @@ def attn_decode_workspace_floats(B, n_heads, head_dim, n_splits):
 
 def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len, out, partial, n_heads, n_kv_heads,
                 head_dim, window, n_splits, lse=None, sinks=None, layout=None, step_max_len=None, seq_order=None,
-                score_bias=None, softcap=0.0, sink_logit=None):
+                score_bias=None, softcap=0.0, sink_logit=None, slopes=None):
     """One query per sequence over the cache pages (laid out as `layout` says, default page_layout(head_dim));
     seq_len counts the new key.  lse as in attn_prefill.  step_max_len (int32 [1] on the device, optional): the
     length of the step's longest sequence, with which sequences of unequal lengths are cut into splits of equal
@@ -669,11 +671,11 @@ def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len,
         library.check(library.lib().yalm_attn_decode_lse(
             p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_ss, p_sl, p_o, p_lse, p_w, B, n_heads, n_kv_heads, head_dim,
             int(window), int(n_splits), n_pages, _layout(layout, head_dim), dtype_code(dt), force, p_max, p_ord,
-            *_bias(score_bias, n_heads), *_shape(softcap, sink_logit, n_heads), _stream()), "attn_decode")
+            *_bias(score_bias, n_heads), *_shape(softcap, sink_logit, n_heads, slopes), _stream()), "attn_decode")
         return out
     if lse is not None:
         raise ValueError("attn_decode leaves no lse when it takes the sinks in itself")
-    if score_bias is not None or softcap or sink_logit is not None:
+    if score_bias is not None or softcap or sink_logit is not None or slopes is not None:
         raise ValueError("attention sinks are scored without a score bias, a cap or a sink logit: they do not go together")
     sink_k, sink_v, cos_sin, rotary_dim, store = sinks
     n_slots, _, n_sinks, _ = sink_k.shape

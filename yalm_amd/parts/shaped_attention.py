@@ -126,6 +126,10 @@ class ShapedAttention(Part):
     def score_bias(self):
         return getattr(self.position, "score_bias", None)
 
+    @property
+    def slopes(self):
+        return getattr(self.position, "slopes", None)
+
     def forward(self, h, x, ctx, line, writes_cache=True):
         T = h.shape[0]
         act, ws = h.dtype, ctx.ws
@@ -158,11 +162,11 @@ class ShapedAttention(Part):
         if prefill:
             kernels.attn_prefill(q, kst, vst, o, ctx.cu_seqlens, seq_tile0, ctx.tok_seq, ctx.tok_pos, H, G, P, self.window,
                                  tiles.get("tile_order"), score_bias=self.score_bias, softcap=self.softcap,
-                                 sink_logit=self.sink)
+                                 sink_logit=self.sink, slopes=self.slopes)
         else:
             n_splits = decode_splits(H, G, P, T, min(group.ring_pages, ctx.pages_bucket), ctx.ragged)
             partial = ws.get("attn.partial", (kernels.attn_decode_workspace_floats(T, H, P, n_splits),), torch.float32)
             kernels.attn_decode(q, k_pages, v_pages, group.table, group.ring_pages, ctx.seq_slot, ctx.seq_len, o, partial,
                                 H, G, P, self.window, n_splits, step_max_len=ctx.step_max_len, seq_order=ctx.seq_order,
-                                score_bias=self.score_bias, softcap=self.softcap, sink_logit=self.sink)
+                                score_bias=self.score_bias, softcap=self.softcap, sink_logit=self.sink, slopes=self.slopes)
         self._gemm(ctx, o, self.wo, x, kernels.EPI_ADD_F32)
