@@ -519,3 +519,53 @@ def test_trace_runner(folders, tmp_path, dtype):
     differ = sum(check_request(got[rid], folders[("mixed", dtype)], dtype, toks, "trace_run %s %s" % (dtype, rid))
                  for rid, toks in requests.items())
     assert differ <= 10
+
+
+# ------------------------------------------------------------------------------------------ configurations drawn at random
+def random_config(seed):
+    """A Gedunex configuration whose every size, count, constant and the order of its layers are drawn from `seed`."""
+    g = np.random.default_rng(seed)
+    pick = lambda lo, hi: int(g.integers(lo, hi + 1))
+    width = pick(17, 150)
+    layers, blend_shape = [], None
+    for _ in range(pick(2, 6)):
+        if g.random() < 0.35:
+            mixer = GC.rec(pick(1, 4), pick(2, 70), pick(2, 70), float(g.uniform(2.0, 20.0)))
+        else:
+            kv = pick(1, 4)
+            heads = kv * pick(1, 5)
+            dim, vdim = pick(2, 72), pick(2, 72)
+            blend = g.random() < 0.5
+            if blend and blend_shape is None:
+                blend_shape = (kv, vdim)
+            elif blend:
+                kv, vdim = blend_shape
+                heads = kv * pick(1, 5)
+            mixer = GC.attn(heads, kv, dim, vdim, float(g.uniform(0.05, 0.5)),
+                            window=pick(1, 130) if g.random() < 0.7 else None,
+                            softcap=float(g.uniform(2.0, 40.0)) if g.random() < 0.7 else None,
+                            q_temp=(float(g.uniform(0.1, 1.0)), pick(1, 90)) if g.random() < 0.6 else None, v_mix=blend)
+        r = g.random()
+        mlp = None if r < 0.15 else GC.dense(pick(5, 200)) if r < 0.5 else None
+        if r >= 0.5:
+            experts = pick(1, 9)
+            mlp = GC.moe(experts, pick(1, experts), pick(3, 60))
+        layers.append(GC.layer(mixer, mlp))
+    return GC.model(pick(30, 400), width, float(10.0 ** g.uniform(-7, -4)), float(g.uniform(0.5, 14.0)), layers)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", [11, 12, 13, 14, 15, 16, 17, 18])
+def test_configurations_drawn_at_random(tmp_path, seed, dtype):
+    """Held to the plain implementation at every position: a whole prompt, a prompt with its last tokens one by one, and
+    two unequal requests in one batch."""
+    from yalm_amd.engine import Engine, Model
+    cfg = random_config(seed)
+    folder = make_folder(tmp_path, "random%d" % seed, cfg, seed, helpers.torch_dtype(dtype))
+    engine = Engine(Model.from_folder(folder, dtype=helpers.torch_dtype(dtype), device=DEV, strict=True), max_tokens=2048)
+    requests = requests_for(cfg, [150, 41], seed=seed)
+    folders = {("r", dtype): folder}
+    compare(folders, "r", dtype, schedules.whole(requests), requests, engine, "random %d whole" % seed)
+    compare(folders, "r", dtype, schedules.tail_one_by_one(requests, tail=60), requests, engine, "random %d tail" % seed)
+    compare(folders, "r", dtype, schedules.batches(requests, [list(requests)], {"r0": 97, "r1": 3}), requests, engine,
+            "random %d batch" % seed)
