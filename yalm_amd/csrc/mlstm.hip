@@ -11,6 +11,7 @@
 // sequence's tokens of the step in order (one in a decode step) and puts the state back.  Threads stand as
 // [row groups][columns]: a thread owns the rows k = group, group + groups, ... of one column of S, so that S needs no
 // synchronisation of its own, and a column's sum over the groups is made through LDS.
+#include <type_traits>
 #include "common.h"
 #include "yalm_hip.h"
 
@@ -293,12 +294,24 @@ __global__ __launch_bounds__(ML_THREADS) void mlstm_chunk_kernel(
       for (int c = 0; c < RT; ++c) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
       const float* qa = Qs + (wave * 16 + lr) * QROW + lq;
       const float* kb = Ks + lr * QROW + lq;
+      // the number of key tiles is the wave's own: a loop of its own for each number, so that none carries a branch
+      // (a branch around every product keeps the loads of the next from being asked for under it)
+      auto products = [&](auto nc) {
 #pragma unroll 4
-      for (int k0 = 0; k0 < d16; k0 += 4) {
-        const float a = qa[k0];
+        for (int k0 = 0; k0 < d16; k0 += 4) {
+          const float a = qa[k0];
 #pragma unroll
-        for (int c = 0; c < RT; ++c)
-          if (c <= wave) acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, kb[c * 16 * QROW + k0], acc[c], 0, 0, 0);
+          for (int c = 0; c < decltype(nc)::value; ++c)
+            acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, kb[c * 16 * QROW + k0], acc[c], 0, 0, 0);
+        }
+      };
+      if constexpr (RT == 4) {
+        if (wave == 0) products(std::integral_constant<int, 1>{});
+        else if (wave == 1) products(std::integral_constant<int, 2>{});
+        else if (wave == 2) products(std::integral_constant<int, 3>{});
+        else products(std::integral_constant<int, 4>{});
+      } else {
+        products(std::integral_constant<int, 1>{});
       }
       float sum[4] = {0.f, 0.f, 0.f, 0.f};        // of the rows lq * 4 + v over this lane's columns
 #pragma unroll
@@ -371,12 +384,21 @@ __global__ __launch_bounds__(ML_THREADS) void mlstm_chunk_kernel(
       }
       const float* ka = Ks + lq * QROW + r0 * 16 + lr;
       const float* vb = Vs + lq * VROW + wave * 16 + lr;
+      if (nr == 4) {                              // the loop without a branch (see the scores' products)
 #pragma unroll 4
-      for (int s0 = 0; s0 < L; s0 += 4) {
-        const float bvv = vb[s0 * VROW], cs = cv[s0 + lq];
+        for (int s0 = 0; s0 < L; s0 += 4) {
+          const float bvv = vb[s0 * VROW], cs = cv[s0 + lq];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if (j < nr) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[s0 * QROW + j * 16] * cs, bvv, acc[j], 0, 0, 0);
+          for (int j = 0; j < 4; ++j)
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[s0 * QROW + j * 16] * cs, bvv, acc[j], 0, 0, 0);
+        }
+      } else {
+        for (int s0 = 0; s0 < L; s0 += 4) {
+          const float bvv = vb[s0 * VROW], cs = cv[s0 + lq];
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (j < nr) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[s0 * QROW + j * 16] * cs, bvv, acc[j], 0, 0, 0);
+        }
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j)
