@@ -113,7 +113,7 @@ KERNEL_FACES = ("embed", "rmsnorm", "gemm", "gemm_norm", "gemm_norm_qkv_rope", "
                 "gemm_chain", "gemm_chain_qkv_rope", "rope_kv_write", "rope_kv_write_tiles", "attn_prefill",
                 "attn_decode", "sink_store", "attn_sink_mix", "argmax", "cast", "norm_add", "polynorm", "head_matmul",
                 "latent_pack", "moe_route", "moe_select", "moe_pair_gate_up", "moe_pair_down", "moe_grouped", "embed_sinusoid",
-                "qkv_pack", "mlstm_scan", "mlstm_chunks")
+                "qkv_pack", "v_tiles", "mlstm_scan", "mlstm_chunks")
 FP32_FACES = ("mlstm_scan", "mlstm_chunks")     # kernels of float32 multiply-adds whatever the model's dtype: priced against that peak
 
 
@@ -200,6 +200,8 @@ def kernel_cost(name, a, kw, kv_tokens, torch):
         T = qkv.shape[0]
         n_kv, pad = a[23], a[26]
         return "qkv_pack %d tokens" % T, nbytes(qkv, q_out) + 2 * T * n_kv * pad * q_out.element_size() * (2 if a[11] is not None else 1), 0.0
+    if name == "v_tiles":
+        return "v_tiles %d tokens" % a[0].shape[0], nbytes(a[0], a[1]) + (nbytes(a[0]) if a[2] is not None else 0), 0.0
     if name == "mlstm_scan":
         proj, state, seq_slot, out = a[0], a[4], a[6], a[7]
         H, d, dv = a[8], a[9], a[10]

@@ -53,15 +53,17 @@ def test_embedding_with_scale_and_sinusoid(D, dtype):
     assert torch.equal(out[0].cpu(), table[2].float() * 0.5) and float(out[1].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("by_tiles", [False, True])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,d,dv,temp,blend", [(2, 1, 8, 6, None, 0), (6, 2, 8, 20, (0.4, 3), 1), (4, 4, 24, 8, (1.0, 1), 2),
                                                  (17, 1, 5, 9, (0.3, 256), 2), (3, 3, 40, 40, None, 0)])
-def test_packing_kernel(dtype, H, G, d, dv, temp, blend):
+def test_packing_kernel(dtype, H, G, d, dv, temp, blend, by_tiles):
     """Biases, whole-projection norms, temperature, blending and the staged keys and values of a step of whole prompts,
-    against the plain projections fed through identity matrices."""
+    against the plain projections fed through identity matrices; the values transposed token by token, or left in rows
+    and transposed a tile at a time."""
     from yalm_amd.ops import kernels
     from yalm_amd.parts.attention import kv_tiles
-    n_tok = [3, 70, 1]
+    n_tok = [3, 70, 1]                            # 74 tokens: enough for the kernel that works a wave a token
     T = sum(n_tok)
     Q, K, V = H * d, G * d, G * dv
     N = Q + K + V
@@ -83,9 +85,15 @@ def test_packing_kernel(dtype, H, G, d, dv, temp, blend):
     vst = torch.full((tiles["n_tiles"], G, pad, 64), float("nan"), dtype=dtype, device=DEV)
     v_first = first.clone().to(DEV)
     bias = torch.cat([w["a.q.b"], w["a.k.b"], w["a.v.b"]]).to(DEV)
+    v_rows = torch.full((T, G * pad), float("nan"), dtype=dtype, device=DEV) if by_tiles else None
     kernels.qkv_pack(raw.to(DEV), bias, w["a.q.norm"].to(DEV), w["a.k.norm"].to(DEV), 1e-5, temp, 1.7, v_first if blend else None,
                      blend, torch.tensor([lam], device=DEV) if blend == 2 else None, q_out, kst, vst, i32(tiles["seq_tile0"]),
-                     None, None, None, 0, i32(np.repeat(np.arange(3), n_tok)), i32(positions), i32([0, 1, 2]), None, H, G, d, dv, pad)
+                     None, None, None, 0, i32(np.repeat(np.arange(3), n_tok)), i32(positions), i32([0, 1, 2]), None, H, G, d, dv, pad,
+                     v_rows=v_rows)
+    if by_tiles:
+        kernels.v_tiles(v_rows, vst, None, i32(np.concatenate([[0], np.cumsum(n_tok)])), i32(tiles["seq_tile0"]), None, 0,
+                        i32([0, 1, 2]), None, G, pad)
+        assert float(vst[0, :, :, 3:].float().abs().sum()) == 0.0      # rows behind a sequence's end are zeros
     q, k, v = P.attention_projections(raw.to(F64), positions, mixer, w, "a.", 1e-5)
     if blend == 2:
         v = (1 - lam) * v + lam * first.to(F64).reshape(T, G, dv)

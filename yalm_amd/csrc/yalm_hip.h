@@ -322,7 +322,13 @@ int yalm_qkv_pack(const float* qkv, const float* bias, const float* w_q, const f
                   void* v_stage, const int* seq_tile0, void* k_pages, void* v_pages, const int* block_table,
                   int table_stride, int ring_pages, const int* tok_seq, const int* tok_pos, const int* seq_slot,
                   const int* seq_len, int T, int n_heads, int n_kv_heads, int d, int dv, int pad, int n_pages,
-                  int page_layout, int dtype, hipStream_t stream);
+                  int page_layout, int dtype, void* v_rows, hipStream_t stream);
+// v_rows (`dtype` [T, G, pad]; may be null): yalm_qkv_pack then leaves the values there row by row instead of in their
+// transposed places, and yalm_v_tiles brings them into v_stage [n_tiles, G, pad, 64] and the cache pages (v_pages null:
+// none) a tile of 64 tokens at a time through LDS (64 (pad + 2) elements must fit 64 KB).
+int yalm_v_tiles(const void* v_rows, void* v_stage, void* v_pages, const int* cu_seqlens, const int* seq_tile0,
+                 const int* block_table, int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, int B,
+                 int n_tiles, int n_kv_heads, int pad, int n_pages, int page_layout, int dtype, hipStream_t stream);
 
 // The matrix-memory recurrence (mlstm.hip): proj float32 [T, 2 H d + 2 H dv + 2 H] = q | k | v | g | z_i | z_f of
 // every token; state float32 [n_slots, H, d dv + d + 1] (S, n, m of every head), read and left advanced; out `dtype`

@@ -848,15 +848,44 @@ def latent_pack(proj, q_head, q_rot_off, kv_off, norm_w, eps, q_scale, out, n_he
     return out
 
 
+def can_v_tiles(pad, dtype):
+    """Whether v_tiles takes heads of this width (a tile of 64 tokens of a head waits in 64 KB of LDS)."""
+    return PAGE * (pad + 2) * (4 if dtype == torch.float32 else 2) <= 64 * 1024
+
+
+def v_tiles(v_rows, v_stage, v_pages, cu_seqlens, seq_tile0, block_table, ring_pages, seq_slot, seq_len, n_kv_heads, pad):
+    """The values that qkv_pack left row by row (v_rows [T, G pad]) into the transposed staging tiles [n_tiles, G, pad,
+    64] and cache pages (None: nowhere) of a step of whole prompts, a tile of 64 tokens at a time."""
+    T = v_rows.shape[0]
+    dt = v_rows.dtype
+    B = seq_slot.shape[0]
+    n_tiles = v_stage.shape[0]
+    if not can_v_tiles(pad, dt):
+        raise ValueError("v_tiles: heads of %d are too wide" % pad)
+    n_pages, stride = 0, 0
+    if v_pages is not None:
+        n_pages, stride = v_pages.shape[0], block_table.shape[1]
+        if ring_pages <= 0 or ring_pages > stride:
+            raise ValueError("ring_pages %d does not fit the block table (%d columns)" % (ring_pages, stride))
+    library.check(library.lib().yalm_v_tiles(
+        _need(v_rows, "v_rows", dt, (T, n_kv_heads * pad)), _need(v_stage, "v_stage", dt, (n_tiles, n_kv_heads, pad, PAGE)),
+        _opt(v_pages, "v_pages", dt, (n_pages, n_kv_heads, pad, PAGE)), _need(cu_seqlens, "cu_seqlens", torch.int32, (B + 1,)),
+        _need(seq_tile0, "seq_tile0", torch.int32, (B + 1,)), _opt(block_table, "block_table", torch.int32, (None, None)), stride,
+        int(ring_pages), _need(seq_slot, "seq_slot", torch.int32, (B,)), _opt(seq_len, "seq_len", torch.int32, (B,)), B, n_tiles,
+        n_kv_heads, pad, n_pages, page_layout(pad), dtype_code(dt), _stream()), "v_tiles")
+    return v_stage
+
+
 def qkv_pack(qkv, bias, w_q, w_k, eps, q_temp, q_scale, v_first, blend, lam, q_out, k_stage, v_stage, seq_tile0, k_pages,
-             v_pages, block_table, ring_pages, tok_seq, tok_pos, seq_slot, seq_len, n_heads, n_kv_heads, d, dv, pad):
+             v_pages, block_table, ring_pages, tok_seq, tok_pos, seq_slot, seq_len, n_heads, n_kv_heads, d, dv, pad,
+             v_rows=None):
     """From a q/k/v product to an attention without rotation.  qkv float32 [T, H d + G d + G dv] (+ bias, float32 of
     that width or None); RMS norms over the WHOLE query and key projections with the weights w_q [H d], w_k [G d]
     (float32; None: no norm); the queries times q_scale and, with q_temp = (coef, every), times 1 + coef ln(floor((p + 1)
     / every) + 1) at position p; blend 1 stores the values in v_first (float32 [T, G dv]), blend 2 replaces them by
     (1 - lam) v + lam v_first (lam: one float32 on the device).  Heads are written `pad` wide, zeros behind: q_out [T,
     H pad]; keys and values into the cache pages (None: nowhere) and, with k_stage, into the staging tiles of a step of
-    whole prompts."""
+    whole prompts.  v_rows ([T, G pad], optional): the values go there row by row instead (v_tiles then transposes them)."""
     T = qkv.shape[0]
     Q, K, V = n_heads * d, n_kv_heads * d, n_kv_heads * dv
     N = Q + K + V
@@ -884,7 +913,7 @@ def qkv_pack(qkv, bias, w_q, w_k, eps, q_temp, q_scale, v_first, blend, lam, q_o
         _opt(v_pages, "v_pages", dt, (n_pages, n_kv_heads, pad, PAGE)), _opt(block_table, "block_table", torch.int32, (None, None)),
         stride, int(ring_pages), _need(tok_seq, "tok_seq", torch.int32, (T,)), _need(tok_pos, "tok_pos", torch.int32, (T,)),
         _need(seq_slot, "seq_slot", torch.int32), _opt(seq_len, "seq_len", torch.int32), T, n_heads, n_kv_heads, d, dv, pad,
-        n_pages, page_layout(pad), dtype_code(dt), _stream()), "qkv_pack")
+        n_pages, page_layout(pad), dtype_code(dt), _opt(v_rows, "v_rows", dt, (T, n_kv_heads * pad)), _stream()), "qkv_pack")
     return q_out
 
 

@@ -64,7 +64,8 @@ _SIGNATURES = {
     "yalm_moe_grouped": (_I, [_P, _P, _P, _P, _P, _P, _F, _F, _F, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_embed_sinusoid": (_I, [_P, _I, _P, _P, _P, _F, _P, _I, _I, _I, _P]),
     "yalm_qkv_pack": (_I, [_P, _P, _P, _P, _F, _F, _I, _F, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P,
-                           _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
+                           _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
+    "yalm_v_tiles": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_mlstm_chunks": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _F, _F, _I, _I, _I, _P]),
     "yalm_mlstm_chunks_lds": (ctypes.c_long, [_I, _I]),
     "yalm_mlstm_scan": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _F, _F, _I, _I, _P]),
@@ -72,7 +73,7 @@ _SIGNATURES = {
     "yalm_probe_mfma": (_I, [_I, _I, _I, _P, _P, _P]),
 }
 
-ABI_VERSION = 31
+ABI_VERSION = 32
 
 
 class KernelError(RuntimeError):

@@ -22,6 +22,10 @@ from ..weights.loader import ParamSpec, place
 from .attention import decode_splits, kv_tiles
 from .base import Part, build_part, part
 
+# A prompt step of at least this many tokens leaves its values row by row and transposes them a tile of 64 tokens at a
+# time (whole lines into the staging tiles and pages instead of two bytes a token and element)
+V_TILES_MIN_TOKENS = 64
+
 NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "out": "o_proj.weight",
          "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "q_norm": "q_norm.weight",
          "k_norm": "k_norm.weight", "sink": "sink", "blend": "value_blend"}
@@ -154,10 +158,16 @@ class ShapedAttention(Part):
             # the first blending layer of a step leaves its values here for the later ones of the same step
             v_first = ws.get("attn.blend." + self.blend_name, (T, self.v_dim), torch.float32)
             blend = 1 if self.value_blend == "first" else 2
+        v_rows = None
+        if prefill and T >= V_TILES_MIN_TOKENS and kernels.can_v_tiles(P, act):
+            v_rows = ws.get("attn.vrows", (T, G * P), act)
         kernels.qkv_pack(qkv, self.bias, self.w_qn, self.w_kn, self.eps, self.q_temp, self.scale * math.sqrt(P), v_first,
                          blend, self.lam, q, kst, vst, seq_tile0, k_pages if writes_cache else None,
                          v_pages if writes_cache else None, group.table, group.ring_pages, ctx.tok_seq, ctx.tok_pos,
-                         ctx.seq_slot, ctx.seq_len, H, G, self.key_dim, self.value_dim, P)
+                         ctx.seq_slot, ctx.seq_len, H, G, self.key_dim, self.value_dim, P, v_rows=v_rows)
+        if v_rows is not None:
+            kernels.v_tiles(v_rows, vst, v_pages if writes_cache else None, ctx.cu_seqlens, seq_tile0, group.table,
+                            group.ring_pages, ctx.seq_slot, ctx.seq_len, G, P)
         o = ws.get("attn.o", (T, H * P), act)
         if prefill:
             kernels.attn_prefill(q, kst, vst, o, ctx.cu_seqlens, seq_tile0, ctx.tok_seq, ctx.tok_pos, H, G, P, self.window,
