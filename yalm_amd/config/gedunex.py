@@ -16,8 +16,8 @@ Tensors: `embed`, `head`, `final.norm`, and for layer i `l<i>.norm1`;
 What the design fixes and this file therefore states: the sinusoid's base 10000; head h of H has the slope
 2^(-8 (h + 1) / H) on the distance of query and key; the recurrence's denominator floor 1e-6 and its query scale
 dim^(-1/2); every norm is an RMS norm with the one eps; the experts are silu(gate) * up and a token's weights are the
-softmax over its chosen logits; the values of every layer with `v_mix` but the first such layer are blended with
-the first one's."""
+softmax over its chosen logits; among the layers with `v_mix` the earliest keeps its own values and hands them to
+the others, which blend theirs with them."""
 from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional
 

@@ -27,7 +27,7 @@ struct ScoreBias {
   const float* table;
   int n;
   float softcap;               // score <- softcap tanh(score / softcap) before the distance's term (0: no cap)
-  const float* sink_logit;     // [heads]: a logit in the softmax's denominator that has no key and no value (null: none)
+  const float* sink_logit;     // [heads]: one more term exp(sink_logit[head]) of the softmax's denominator, without a key (null: none)
   const float* slope;          // [heads]: -slope[head] * distance is added to every score (null: none)
   __device__ __forceinline__ float at(int head, int distance) const {
     float term = table != nullptr ? table[(size_t)head * n + min(max(distance, 0), n - 1)] : 0.f;

@@ -1,5 +1,5 @@
 // The matrix-memory recurrence (mLSTM) of a head: a state S [d, dv], a vector n [d] and a running maximum m per
-// sequence and head, all float32, carried from token to token.
+// sequence and head, all float32, kept from one step of the sequence to the next.
 //
 //   i = cap tanh((z_i + b_i) / cap),  f = logsigmoid(cap tanh((z_f + b_f) / cap))          (cap 0: uncapped)
 //   m' = max(f + m, i);  S' = exp(f + m - m') S + exp(i - m') k v^T;  n' likewise with k alone

@@ -244,8 +244,10 @@ __global__ __launch_bounds__(VT_THREADS) void v_tiles_kernel(
     const int* __restrict__ seq_tile0, const int* __restrict__ block_table, int table_stride, int ring_pages,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_len, int B, int n_kv_heads, int pad, int n_pages,
     int page_layout) {
+  constexpr int VEC = 16 / sizeof(T);             // elements of a 16-byte access (pad is a multiple of 16)
+  struct __attribute__((aligned(16))) Chunk { T v[VEC]; };
   extern __shared__ __attribute__((aligned(16))) unsigned char vt_raw[];
-  T* tl = reinterpret_cast<T*>(vt_raw);           // [PAGE][pad + 2]
+  T* tl = reinterpret_cast<T*>(vt_raw);           // [PAGE][pad + VEC]
   const int tile = blockIdx.x, g = blockIdx.y, tid = threadIdx.x;
   int lo = 0, hi = B - 1;
   while (lo < hi) {
@@ -255,10 +257,15 @@ __global__ __launch_bounds__(VT_THREADS) void v_tiles_kernel(
   const int b = lo, tq = tile - seq_tile0[b];
   const int start = cu_seqlens[b], len = cu_seqlens[b + 1] - start;
   const int n_rows = min(PAGE, len - tq * PAGE);
-  const int row_w = pad + 2;
-  for (int i = tid; i < PAGE * pad; i += VT_THREADS) {
-    const int r = i / pad, e = i - r * pad;
-    tl[r * row_w + e] = r < n_rows ? v_rows[((size_t)(start + tq * PAGE + r) * n_kv_heads + g) * pad + e] : from_f32<T>(0.f);
+  const int row_w = pad + VEC, per_row = pad / VEC;
+  for (int i = tid; i < PAGE * per_row; i += VT_THREADS) {
+    const int r = i / per_row, c = i - r * per_row;
+    Chunk ch;
+#pragma unroll
+    for (int u = 0; u < VEC; ++u) ch.v[u] = from_f32<T>(0.f);
+    if (r < n_rows)
+      ch = *reinterpret_cast<const Chunk*>(v_rows + ((size_t)(start + tq * PAGE + r) * n_kv_heads + g) * pad + c * VEC);
+    *reinterpret_cast<Chunk*>(tl + r * row_w + c * VEC) = ch;
   }
   __syncthreads();
   T* vp = nullptr;
@@ -271,11 +278,16 @@ __global__ __launch_bounds__(VT_THREADS) void v_tiles_kernel(
     }
   }
   T* vs = v_stage + ((size_t)tile * n_kv_heads + g) * PAGE * pad;
-  for (int i = tid; i < PAGE * pad; i += VT_THREADS) {
-    const int e = i / PAGE, r = i % PAGE;
-    const T v = tl[r * row_w + e];
-    vs[(size_t)e * PAGE + r] = v;                 // rows behind the sequence's end are zeros
-    if (vp != nullptr && r < n_rows) vp[page_v_offset(page_layout, r, e, pad)] = v;
+  constexpr int RC = PAGE / VEC;                  // runs of VEC consecutive rows in a tile
+  for (int i = tid; i < pad * RC; i += VT_THREADS) {
+    const int e = i / RC, r0 = (i % RC) * VEC;
+    Chunk ch;
+#pragma unroll
+    for (int u = 0; u < VEC; ++u) ch.v[u] = tl[(r0 + u) * row_w + e];
+    *reinterpret_cast<Chunk*>(vs + (size_t)e * PAGE + r0) = ch;      // rows behind the sequence's end are zeros
+    // a run of consecutive rows lies together in either page layout; rows behind the end belong to tokens still to
+    // come, which write them before anyone reads them
+    if (vp != nullptr && r0 < n_rows) *reinterpret_cast<Chunk*>(vp + page_v_offset(page_layout, r0, e, pad)) = ch;
   }
 }
 }  // namespace
@@ -290,7 +302,8 @@ extern "C" int yalm_v_tiles(const void* v_rows, void* v_stage, void* v_pages, co
       (v_pages != nullptr && (block_table == nullptr || ring_pages <= 0 || seq_len == nullptr)) ||
       !page_layout_ok(page_layout, pad) || (dtype != YALM_F32 && dtype != YALM_BF16))
     return YALM_ERR_ARG;
-  const size_t lds = (size_t)PAGE * (pad + 2) * (dtype == YALM_F32 ? 4 : 2);
+  if (pad % 16 != 0 || ((((uintptr_t)v_rows) | ((uintptr_t)v_stage) | ((uintptr_t)v_pages)) & 15)) return YALM_ERR_ARG;
+  const size_t lds = (size_t)PAGE * (pad + (dtype == YALM_F32 ? 4 : 8)) * (dtype == YALM_F32 ? 4 : 2);
   if (lds > 64 * 1024) return YALM_ERR_ARG;
   dim3 grid(n_tiles, n_kv_heads);
   if (dtype == YALM_F32)

@@ -8,8 +8,8 @@
 
 // What shapes a score between the product q . k / sqrt(head size) and the softmax, beside the mask: a cap
 // (score <- cap tanh(score / cap); 0: none), then a term by the distance of query and key, bias[head][min(distance,
-// n_bias - 1)] (null: none), and a learned logit per head that stands in the softmax's denominator without a key or a
-// value of its own (sink_logit[head], null: none; it is neither scaled nor capped and gets no distance term).
+// n_bias - 1)] (null: none) and/or -slope[head] * distance (null: none), and a logit per head that stands in the
+// softmax's denominator without a key or a value of its own (sink_logit[head], null: none; it enters as it is).
 struct ScoreShape {
   const float* bias;
   int n_bias;

@@ -166,8 +166,8 @@ long yalm_attn_decode_workspace(int B, int n_heads, int head_dim, int n_splits);
 // scaling) by the distance between query and key, score_bias[head, min(distance, n_bias - 1)]: what a position
 // encoding that is no rotation needs (not together with attention sinks).
 // softcap (0: none): score <- softcap tanh(score / softcap), after the scaling and before score_bias's term.
-// sink_logit (device, float32 [n_heads]; may be null): a learned logit per head that counts once in the softmax's
-// denominator and has no key and no value (it is not scaled, not capped and gets no distance term; lse counts it).
+// sink_logit (device, float32 [n_heads]; may be null): one more term exp(sink_logit[head]) of the softmax's denominator,
+// to which no key and no row of values belongs (scale, cap and distance term shape the keys' scores only; lse holds it).
 // slopes (device, float32 [n_heads]; may be null): -slopes[head] * distance is added to every score, as score_bias's
 // term is, without a table.
 int yalm_attn_prefill_lse(const void* q, const void* k_stage, const void* v_stage, void* out, float* out_f32, float* lse,
@@ -325,7 +325,7 @@ int yalm_qkv_pack(const float* qkv, const float* bias, const float* w_q, const f
                   int page_layout, int dtype, void* v_rows, hipStream_t stream);
 // v_rows (`dtype` [T, G, pad]; may be null): yalm_qkv_pack then leaves the values there row by row instead of in their
 // transposed places, and yalm_v_tiles brings them into v_stage [n_tiles, G, pad, 64] and the cache pages (v_pages null:
-// none) a tile of 64 tokens at a time through LDS (64 (pad + 2) elements must fit 64 KB).
+// none) a tile of 64 tokens at a time through LDS (pad a multiple of 16; 64 (pad + 8) elements must fit 64 KB).
 int yalm_v_tiles(const void* v_rows, void* v_stage, void* v_pages, const int* cu_seqlens, const int* seq_tile0,
                  const int* block_table, int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, int B,
                  int n_tiles, int n_kv_heads, int pad, int n_pages, int page_layout, int dtype, hipStream_t stream);

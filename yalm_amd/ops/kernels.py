@@ -582,8 +582,8 @@ def _bias(score_bias, n_heads):
 
 def _shape(softcap, sink_logit, n_heads, slopes=None):
     """(cap, address of the sink logits, address of the slopes): softcap > 0 replaces every scaled score s by softcap
-    tanh(s / softcap) before the score bias; sink_logit, float32 [n_heads] on the device, is a logit per head that counts
-    once in the softmax's denominator and has neither key nor value; slopes, float32 [n_heads] on the device, adds
+    tanh(s / softcap) before the score bias; sink_logit, float32 [n_heads] on the device, puts one more term exp(sink_logit[head]) into the
+    softmax's denominator, a term to which no key and no row of values belongs; slopes, float32 [n_heads] on the device, adds
     -slopes[head] * (query position - key position) to every score (what a score_bias table of slope times distance
     would add, without the table)."""
     cap = float(softcap or 0.0)
@@ -850,7 +850,7 @@ def latent_pack(proj, q_head, q_rot_off, kv_off, norm_w, eps, q_scale, out, n_he
 
 def can_v_tiles(pad, dtype):
     """Whether v_tiles takes heads of this width (a tile of 64 tokens of a head waits in 64 KB of LDS)."""
-    return PAGE * (pad + 2) * (4 if dtype == torch.float32 else 2) <= 64 * 1024
+    return pad % 16 == 0 and PAGE * (pad + 8) * (4 if dtype == torch.float32 else 2) <= 64 * 1024
 
 
 def v_tiles(v_rows, v_stage, v_pages, cu_seqlens, seq_tile0, block_table, ring_pages, seq_slot, seq_len, n_kv_heads, pad):

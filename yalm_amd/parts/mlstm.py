@@ -1,5 +1,5 @@
 """The matrix-memory recurrence of xLSTM (mLSTM) as a mixer: per head a state S [d, dv], a vector n [d] and a
-running maximum m, all float32 and all starting at zero, carried from token to token in the cache's fixed-size
+running maximum m, all float32, zero for a new sequence and kept from one step to the next in the cache's fixed-size
 per-sequence state.
 
 Per token and head: q = W_q h * q_scale, k = W_k h, v = W_v h; i = cap tanh((W_i h + b_i) / cap),
